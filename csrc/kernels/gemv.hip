@@ -649,7 +649,7 @@ static int flight_ks(int need, int tiles, int bz) {
 
 // VGPRs a K-split flight instantiation needs (weight tile + activation / norm registers + ~24 of
 // addressing, accumulators and the prefetch register) against the 512 / KS per lane that KS waves per
-// SIMD leave. Calibrated on the built code objects (tests/test_isa.py): the Q8_0 / Q6_K LayerNorm
+// SIMD leave. Calibrated on the compiler's resource report (scripts/kres.py): the Q8_0 / Q6_K LayerNorm
 // variants above budget (KS = 4 NSB = 1, KS = 2 NSB = 2) were the only ones spilling to scratch.
 template <int QT, int NSB, int KS, int NRM>
 constexpr bool flight_ks_fits() {

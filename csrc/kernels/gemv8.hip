@@ -155,7 +155,7 @@ bool covered(const GemvParams& P, Geo& G) {
   if (in == IN_X8_LN && (G.ks > 2 || (G.nsb == 2 && G.J == 2))) return false;
   // two super-blocks per lane at a 3-4 way K split (K > 16384): the plain image in (down), batch 1; at
   // the 4-way split (1024 threads, <= 128 VGPRs) only the Q4_0 / Q4_K tiles fit without spilling
-  // (tests/test_isa.py)
+  // (the compiler's resource report, scripts/kres.py)
   if (G.nsb == 2 && G.ks > 1 &&
       (in != IN_X8 || (em != EM_ADD && em != EM_NONE) || P.B > 1 || (G.ks == 4 && q != QT_Q4_0 && q != QT_Q4_K)))
     return false;

@@ -7,8 +7,8 @@ namespace omx {
 // Epilogue operands, loaded at block entry ahead of the activation image and the weight stream. The
 // epilogues used to read them after the tile: the residual and the next norm's weight (EM_ADD), the
 // bias, and RoPE's position / frequency plus the KV slot (EPI_QKV) -- each a dependent round trip at
-// the block's tail, several in series behind branch-local vmcnt(0) waits (disassembly of the QKV
-// GEMV: five load + vmcnt(0) pairs after the last dot product). Lane s of a row group writes batch
+// the block's tail, several in series behind branch-local waits (the QKV GEMV had five dependent
+// loads after its last dot product). Lane s of a row group writes batch
 // row b = s (BT rows), so a lane's position / slot are those of row min(s, B - 1).
 template <int J, int BT>
 struct EpiPre {

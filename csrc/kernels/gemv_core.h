@@ -60,9 +60,9 @@ struct WTile {
 #define OMX_PIECE_ORDER() __builtin_amdgcn_sched_barrier(0x0104)
 
 // A sched_barrier only binds the machine scheduler: the SelectionDAG scheduler that runs before it
-// still hoists pure VALU across it, and did -- the disassembly of the K-split down GEMV showed every
-// piece's nibble masks hoisted to the top of the tile, behind ONE s_waitcnt vmcnt(0), so no dot
-// product started before the block's last weight byte had landed (Q6_K: vmcnt(3) after piece 0).
+// still hoists pure VALU across it, and did -- in the K-split down GEMV every piece's nibble masks were
+// hoisted to the top of the tile, behind one wait for all loads, so no dot product started before the
+// block's last weight byte had landed.
 // pin() redefines a loaded register through an empty volatile asm at the point where its piece is
 // consumed: volatile asm statements keep program order, nothing that reads the value can move above
 // its pin, and the waitcnt pass places that load's (counted) vmcnt wait right there.

@@ -2,8 +2,6 @@
 §2.1 R29). Python: compiles, no unused imports (ast), no tabs / trailing whitespace, <= 140 columns.
 HIP/C++ (csrc/): no tabs / trailing whitespace, <= 140 columns, and the MI355X-only policy:
   * no CUDA compatibility layers (cuda_runtime, __CUDA_ARCH__, __HIP_PLATFORM_* dual paths, hipify).
-The scalar-memory policy is enforced on the *built* ISA by an allow-list (scripts/isa_check.py), so
-no source file needs to spell out the instructions it rejects.
 Usage: python scripts/lint.py [paths...]   (exit 1 on findings)"""
 from __future__ import annotations
 
