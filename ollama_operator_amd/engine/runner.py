@@ -28,7 +28,7 @@ from ..ops.reference import TorchExecutor
 from ..utils.trace import trace_range
 from .kv_cache import PagedKV
 from .sampling import SamplingOptions, sample_host
-from .weights import DeviceWeights, DevQMat
+from .weights import DeviceWeights, DevQMat, StackWeights
 
 HIST_CAP = 256
 GEMM_SPLIT_WS_FLOATS = 32 << 20  # 128 MiB of fp32 split-K slabs (2-way split of a 2048 x 8192 output)
@@ -137,11 +137,12 @@ class Runner:
     def __init__(self, model_path: str, device: str | None = None, max_batch: int = 64, max_seqs: int = 4,
                  ctx: int | None = None, block_size: int = 16, tp_rank: int = 0, tp_size: int = 1,
                  tp_group=None, use_graphs: bool | None = None, weights: DeviceWeights | None = None,
-                 tp_ctrl=None, cpu_backend: str | None = None, ext_rows: int = 0):
+                 tp_ctrl=None, cpu_backend: str | None = None, ext_rows: int = 0, kv_tokens: int = 0):
         """cpu_backend (device "cpu" only): "native" = the quantised C++ backend (csrc/cpu, the serving
         default), "torch" = the fp32 torch twin (test oracle). Default: $OMX_CPU_BACKEND, else native
         when its module is built. ext_rows: capacity of the external embedding rows (image patches of
-        multimodal prompts, `set_ext`); 0 = text only."""
+        multimodal prompts, `set_ext`); 0 = text only. kv_tokens: tokens the KV block pool holds for all
+        live sequences together (each rounded up to whole blocks); 0 = every slot at full context."""
         t0 = time.perf_counter()
         if device is None:
             device = f"cuda:{torch.cuda.current_device()}" if torch.cuda.is_available() else "cpu"
@@ -179,7 +180,7 @@ class Runner:
         self.block_size = block_size
         self.ctx = min(ctx or cfg.ctx_len, cfg.ctx_len)
         self.max_blocks = (self.ctx + block_size - 1) // block_size
-        n_blocks = max_seqs * self.max_blocks
+        n_blocks = self.pool_blocks(kv_tokens)
         dev = self.device
         f32 = dict(device=dev, dtype=torch.float32)
         i32 = dict(device=dev, dtype=torch.int32)
@@ -260,33 +261,7 @@ class Runner:
         ws = max(self._ws_floats(B) for B in range(1, max_batch + 1))
         self.attn_ws = torch.zeros(max(ws, 1), **f32)
         self.attn_cnt = torch.zeros(max_batch * loc["H"], **i32)  # self re-arming tickets
-        self.logits = torch.zeros(max_batch, Vl, **f32)
-        self.full_logits = torch.zeros(max_batch, cfg.n_vocab, **f32) if tp_size > 1 else self.logits
-        # step inputs, packed so one H2D copy refreshes (pos, slot, q_len, q_seq, logit_idx)
-        self.d_step = torch.zeros(6, max_batch, **i32)
-        self.d_pos, self.d_slot, self.d_qlen, self.d_qseq, self.d_logit_idx, self.d_tokens = self.d_step.unbind(0)
-        self.d_block_table = torch.zeros(max_seqs, self.max_blocks, **i32)
-        # sampler state (indexed by batch row)
-        self.s_temp = torch.zeros(max_batch, **f32)
-        self.s_topk = torch.zeros(max_batch, **i32)
-        self.s_topp = torch.ones(max_batch, **f32)
-        self.s_minp = torch.zeros(max_batch, **f32)
-        self.s_rpen = torch.ones(max_batch, **f32)
-        self.s_ppen = torch.zeros(max_batch, **f32)
-        self.s_fpen = torch.zeros(max_batch, **f32)
-        self.s_lastn = torch.zeros(max_batch, **i32)
-        self.s_seed = torch.zeros(max_batch, device=dev, dtype=torch.int64)
-        self.s_step = torch.zeros(max_batch, **i32)
-        self.s_hist = torch.zeros(max_batch, HIST_CAP, **i32)
-        self.s_hcount = torch.zeros(max_batch, **i32)
-        self.s_out = torch.zeros(max_batch, **i32)
-        # multi-block sampler: per-row candidate lists (ceil(V/1024) blocks x 64 x {value, index})
-        # and hand-off tickets (zeroed once; the kernel re-arms them)
-        self.s_ws = torch.zeros(max_batch, -(-cfg.n_vocab // 1024) * 128, **f32)
-        self.s_tickets = torch.zeros(max_batch, **i32)
-        # sampler error word: a row whose logits were non-finite (its id is clamped to 0 on device)
-        self.s_err = torch.zeros(1, **i32)
-        self.kv = PagedKV(n_blocks, block_size, max_seqs, self.max_blocks)
+        self._alloc_step_state(Vl, n_blocks)
         # deferred flash-decode merge (B == 1): attention leaves S <= 8 partial slabs, the O GEMV
         # merges them in its activation prologue (no in-launch ticket + re-read)
         self.defer_kps = int(os.environ.get("OMX_DEFER_KPS", "128"))
@@ -351,6 +326,57 @@ class Runner:
             use_graphs = (self.is_gpu and (tp_size == 1 or self.ar is not None) and
                           os.environ.get("OMX_NO_GRAPH", "0") != "1")
         self.use_graphs = use_graphs
+        self._alloc_host_side()
+        self.load_s = time.perf_counter() - t0
+
+    def pool_blocks(self, kv_tokens: int) -> int:
+        """Blocks of the shared KV pool: every slot at full context, or `kv_tokens` tokens in all."""
+        if kv_tokens > 0:
+            return min(self.max_seqs * self.max_blocks, (kv_tokens + self.block_size - 1) // self.block_size)
+        return self.max_seqs * self.max_blocks
+
+    def _alloc_step_state(self, Vl: int, n_blocks: int) -> None:
+        """Logits, the packed step inputs, the block table, the per-row sampler state and the paged-cache
+        bookkeeping: what every model's step, sampler and scheduler share."""
+        cfg, dev = self.cfg, self.device
+        max_batch, max_seqs, tp_size = self.max_batch, self.max_seqs, self.tp_size
+        f32 = dict(device=dev, dtype=torch.float32)
+        i32 = dict(device=dev, dtype=torch.int32)
+        self.logits = torch.zeros(max_batch, Vl, **f32)
+        self.full_logits = torch.zeros(max_batch, cfg.n_vocab, **f32) if tp_size > 1 else self.logits
+        # step inputs, packed so one H2D copy refreshes (pos, slot, q_len, q_seq, logit_idx)
+        self.d_step = torch.zeros(6, max_batch, **i32)
+        self.d_pos, self.d_slot, self.d_qlen, self.d_qseq, self.d_logit_idx, self.d_tokens = self.d_step.unbind(0)
+        self.d_block_table = torch.zeros(max_seqs, self.max_blocks, **i32)
+        # sampler state (indexed by batch row)
+        self.s_temp = torch.zeros(max_batch, **f32)
+        self.s_topk = torch.zeros(max_batch, **i32)
+        self.s_topp = torch.ones(max_batch, **f32)
+        self.s_minp = torch.zeros(max_batch, **f32)
+        self.s_rpen = torch.ones(max_batch, **f32)
+        self.s_ppen = torch.zeros(max_batch, **f32)
+        self.s_fpen = torch.zeros(max_batch, **f32)
+        self.s_lastn = torch.zeros(max_batch, **i32)
+        self.s_seed = torch.zeros(max_batch, device=dev, dtype=torch.int64)
+        self.s_step = torch.zeros(max_batch, **i32)
+        self.s_hist = torch.zeros(max_batch, HIST_CAP, **i32)
+        self.s_hcount = torch.zeros(max_batch, **i32)
+        self.s_out = torch.zeros(max_batch, **i32)
+        # multi-block sampler: per-row candidate lists (ceil(V/1024) blocks x 64 x {value, index})
+        # and hand-off tickets (zeroed once; the kernel re-arms them)
+        self.s_ws = torch.zeros(max_batch, -(-cfg.n_vocab // 1024) * 128, **f32)
+        self.s_tickets = torch.zeros(max_batch, **i32)
+        # sampler error word: a row whose logits were non-finite (its id is clamped to 0 on device)
+        self.s_err = torch.zeros(1, **i32)
+        self.kv = PagedKV(n_blocks, self.block_size, max_seqs, self.max_blocks)
+
+    def _sampler_module(self):
+        """The native module whose `sample` / `host_alloc_mapped` this runner's steps use."""
+        return native()
+
+    def _alloc_host_side(self) -> None:
+        """Decode graphs, pinned upload buffers and the host-mapped token ring."""
+        max_batch = self.max_batch
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self._host_sampler: dict[int, tuple] = {}
         self._pinned = None
@@ -361,11 +387,10 @@ class Runner:
             # sampled tokens of the B == 1 steps, written by the feedback kernel straight into host-mapped
             # pinned memory (slot = input position % ring): no D2H copy command per step
             self._ring_n = 32  # > the steps in flight: two groups of decode_group steps (generate)
-            h, d = native().host_alloc_mapped(4 * self._ring_n)
+            h, d = self._sampler_module().host_alloc_mapped(4 * self._ring_n)
             self._host_ring_dev = d
             self._host_ring = np.ctypeslib.as_array((ctypes.c_int32 * self._ring_n).from_address(h))
-            weakref.finalize(self, native().host_free_mapped, h)
-        self.load_s = time.perf_counter() - t0
+            weakref.finalize(self, self._sampler_module().host_free_mapped, h)
 
     def close(self) -> None:
         """Release the TP collective workspace (all ranks call this together). The executor forgets
@@ -387,11 +412,11 @@ class Runner:
         self._closed = True
         self.graphs.clear()
         ex, self.exe = self.exe, None
-        if isinstance(ex, NativeExec):
+        if hasattr(ex, "exe"):
             ex.r = None
             ex.exe = None
         for k, v in list(vars(self).items()):  # device buffers and weights: dropped now, not at collection
-            if isinstance(v, (torch.Tensor, list, dict, DeviceWeights)) and k not in ("graphs",):
+            if isinstance(v, (torch.Tensor, list, dict, DeviceWeights, StackWeights)) and k not in ("graphs",):
                 setattr(self, k, None)
         if self.is_gpu:
             torch.cuda.synchronize(self.device)
@@ -567,18 +592,19 @@ class Runner:
             for c0 in range(0, len(tokens), self.max_batch):
                 chunk = tokens[c0:c0 + self.max_batch]
                 self.prefill(sid, chunk, want_logits=False)
-                h = self.resid[:len(chunk)].float()
-                if self.cfg.arch == "phi2":
-                    h = torch.nn.functional.layer_norm(h, (h.shape[-1],), self.w.out_norm, self.w.out_norm_b,
-                                                       self.cfg.norm_eps)
-                else:
-                    h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.cfg.norm_eps) * self.w.out_norm
-                s = h.sum(0)
+                s = self._output_norm(self.resid[:len(chunk)].float()).sum(0)
                 acc = s if acc is None else acc + s
                 n += len(chunk)
             return (acc / max(n, 1)).cpu().numpy()
         finally:
             self.free_sequence(sid)
+
+    def _output_norm(self, h: torch.Tensor) -> torch.Tensor:
+        """The model's final norm over residual rows (embeddings endpoint)."""
+        if self.cfg.arch == "phi2":
+            return torch.nn.functional.layer_norm(h, (h.shape[-1],), self.w.out_norm, self.w.out_norm_b,
+                                                  self.cfg.norm_eps)
+        return h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.cfg.norm_eps) * self.w.out_norm
 
     # ------------------------------------------------------------------ sampling
     def _set_sampler(self, row: int, o: SamplingOptions, history: list[int], seed: int, step: int = 0):
@@ -618,7 +644,7 @@ class Runner:
                          fb_max_blocks=self.max_blocks, fb_bs=self.block_size,
                          fb_host_ring=self._host_ring_dev if B == 1 else 0, fb_ring=self._ring_n,
                          fb_sysfence=self.ring_fence)
-            native().sample(d, stream_handle())
+            self._sampler_module().sample(d, stream_handle())
         else:
             for b in range(B):
                 o, hist, seed, step = self._host_sampler[b]
@@ -911,6 +937,64 @@ class Runner:
         self._sample(n)
         return [int(t) for t in self.s_out[:n].tolist()]
 
+    def step_entries(self, entries: list[tuple]) -> torch.Tensor:
+        """Teacher-forced step: entries[i] = (sid, tokens, want). Every entry's tokens are appended to its
+        sequence in ONE forward (portions of prompts beside single decode tokens, as the scheduler's
+        interleaved admission mixes them), nothing is sampled, and the logits at the `want` places (indices
+        into that entry's tokens) come back as [n_want, n_vocab] in entry order. More rows than max_batch
+        run as several forwards over consecutive rows."""
+        rows = []  # (sid, position, token, wanted)
+        for sid, tokens, want in entries:
+            s = self.kv.seqs[sid]
+            start, n = s.length, len(tokens)
+            if start + n > self.ctx:
+                raise ValueError(f"context overflow: {start + n} > {self.ctx}")
+            self.kv.reserve(sid, start + n)
+            self._sync_block_table(sid)
+            ws = set(int(i) for i in want)
+            if any(i < 0 or i >= n for i in ws):
+                raise ValueError("a wanted place lies outside the entry's tokens")
+            rows += [(sid, start + i, tokens[i], i in ws) for i in range(n)]
+        out = []
+        seg_exe = getattr(getattr(self.exe, "exe", None), "set_segments", None) if self.is_gpu else None
+        for r0 in range(0, len(rows), self.max_batch):
+            part = rows[r0:r0 + self.max_batch]
+            B = len(part)
+            pos = np.asarray([p for _, p, _, _ in part], np.int32)
+            slot = np.asarray([self.kv.slot(sid, p) for sid, p, _, _ in part], np.int32)
+            qseq = np.asarray([self.kv.seqs[sid].row for sid, _, _, _ in part], np.int32)
+            wanted = [i for i, r in enumerate(part) if r[3]]
+            lidx = np.zeros(B, np.int32)
+            lidx[:len(wanted)] = wanted
+            self._upload(np.stack([pos, slot, pos + 1, qseq, lidx]).astype(np.int32),
+                         self._device_tokens([t for _, _, t, _ in part]))
+            with trace_range(f"step_entries rows={B}"):
+                if seg_exe is not None:  # one MFMA flash segment per sequence's contiguous rows
+                    segs, a = [], 0
+                    for i in range(1, B + 1):
+                        if i == B or part[i][0] != part[a][0]:
+                            segs.append((a, i - a))
+                            a = i
+                    seg_exe(segs)
+                    try:
+                        self.forward(B, len(wanted), use_idx=True, prefill=True)
+                    finally:
+                        seg_exe([])
+                else:
+                    self.forward(B, len(wanted), use_idx=True, prefill=False)
+            if wanted:
+                out.append(self.full_logits[:len(wanted), :self.cfg.n_vocab].float().clone())
+        for sid, tokens, _ in entries:
+            self.kv.seqs[sid].tokens.extend(tokens)
+        if not out:
+            return torch.zeros(0, self.cfg.n_vocab, device=self.device)
+        return torch.cat(out, 0)
+
+    def reusable_prefix(self, sid: int, n: int) -> int:
+        """How many of the `n` leading tokens that sequence `sid` shares with a new prompt can be kept.
+        A paged KV cache can be cut back to any length; a model with recurrent state overrides this."""
+        return n
+
     def recompose(self, rows: list[tuple], tokens: list[int]) -> None:
         """New batch composition: rows[b] = (opts, history, seed, n_sampled) and the rows' next inputs."""
         for b, (o, hist, seed, n) in enumerate(rows):
@@ -1006,8 +1090,8 @@ class Runner:
         seed = o.resolved_seed()
         st = self.kv.seqs[sid]
         keep = self.kv.common_prefix(st.tokens, prompt)
-        keep = min(keep, len(prompt) - 1)
-        self.kv.truncate(sid, keep)
+        keep = self.reusable_prefix(sid, min(keep, len(prompt) - 1))
+        self._keep_prefix(sid, keep, prompt)
         t0 = time.perf_counter()
         self.prefill(sid, prompt[keep:])
         self._set_sampler(0, o, prompt, seed)

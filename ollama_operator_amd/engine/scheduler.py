@@ -243,6 +243,7 @@ class BatchScheduler:
         best, keep = None, -1
         for sid in self.idle:
             n = kv.common_prefix(kv.seqs[sid].tokens, prompt)
+            n = self.r.reusable_prefix(sid, min(n, len(prompt) - 1))
             if n > keep:
                 best, keep = sid, n
         if best is not None and keep > 0:

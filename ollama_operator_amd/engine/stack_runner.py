@@ -1,0 +1,207 @@
+"""Runner of layer-list models (models/config.py StackConfig): heterogeneous layers, each with its own
+sequence mixer (paged softmax attention, or retention with a per-sequence state matrix) and a routed
+feed-forward, optionally with a span of layers that runs several times over the same weights.
+
+`StackRunner` is a `Runner`: sequences, the paged block pool, prefill chunking, batched admission, decode
+graphs, the sampler and the scheduler interface are the base class's. What differs is what a step runs
+(`forward`: the stack executor, csrc/stack) and what a sequence owns:
+
+* every layer RUN (a repeated layer counts once per pass) has its own cache: attention runs share the
+  sequence's block table and own a K and a V pool [blocks][kv_heads][block][dim | vdim]; retention runs own
+  a float32 state [slots][heads][dim][vdim], indexed by the sequence's block-table row (its slot);
+* a slot's states are cleared when a sequence takes it, and a sequence with state keeps a cached prefix
+  only whole (a state cannot be cut back), never a shorter one;
+* the residual stream is float32; matrices and the K/V pools are bfloat16 (`dtype="bfloat16"`) or
+  float32 (`dtype="float32"`: everything exact, FMA matrix products).
+
+On a GPU the executor is the HIP one and nothing else; the torch twin (ops/reference.py
+TorchStackExecutor) runs the same buffers on the CPU for the host-logic tests.
+"""
+from __future__ import annotations
+
+import os
+import time
+
+import torch
+
+from ..models.config import MIX_ATTENTION, MIX_RETENTION
+from .runner import Runner
+from .weights import StackWeights
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32}
+
+
+class StackExec:
+    """Adapter: runner buffers -> the native stack executor (`_stack.Executor`, csrc/stack)."""
+
+    def __init__(self, r: "StackRunner"):
+        from ..ops import stack_native
+        C = stack_native()
+        self.r = r
+        self.exe = e = C.Executor()
+        w, cfg = r.w, r.cfg
+        p = lambda t: t.data_ptr() if t is not None else 0  # noqa: E731
+        e.configure(dict(E=cfg.n_embd, V=cfg.n_vocab, eps=float(cfg.norm_eps), residual_mult=float(cfg.residual_mult),
+                         logit_softcap=float(cfg.logit_softcap), f32=int(w.dtype == torch.float32),
+                         max_B=r.max_batch, max_seqs=r.max_seqs))
+        e.set_globals(dict(embed=p(w.embed), loop_in=p(w.loop_in), final_w=p(w.final_w), final_b=p(w.final_b),
+                           head=p(w.head)))
+        for i, (L, spec) in enumerate(zip(w.layers, cfg.layers)):
+            m, f = spec.mixer, spec.mlp
+            d = dict(kind=m.kind, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale,
+                     softcap=m.softcap, qtemp_coef=m.qtemp_coef, qtemp_every=m.qtemp_every, rot_dims=m.rot_dims,
+                     n_in=L["n_in"], norm_w=p(L["norm_w"]), norm_b=p(L["norm_b"]), w_in=p(L["w_in"]), w_o=p(L["w_o"]),
+                     decay=p(L.get("decay")), inv_freq=p(L.get("inv_freq")),
+                     **{"off_" + k: v for k, v in L["off"].items()})
+            if f is not None:
+                d.update(experts=f.experts, top=f.top, ff=f.ff, shared_ff=f.shared_ff, router_b=p(L["router_b"]),
+                         w_gu=p(L["w_gu"]), w_down=p(L["w_down"]), sh_down=p(L.get("sh_down")))
+            e.set_layer(i, d)
+        e.set_runs([dict(layer=li, opens_pass=int(first), kc=p(r.kc[ri]), vc=p(r.vc[ri]), state=p(r.states[ri]))
+                    for ri, (li, _ps, first) in enumerate(r.runs)])
+        e.set_workspace(dict(resid=p(r.resid), x0=p(r.x0), h=p(r.hbuf), cat=p(r.catbuf), proj=p(r.proj),
+                             ld_proj=r.proj.shape[1], a=p(r.abuf), ld_a=r.abuf.shape[1], hmid=p(r.hmid),
+                             ld_hmid=r.hmid.shape[1], y=p(r.ybuf), eids=p(r.eids), ew=p(r.ew), ld_top=r.eids.shape[1],
+                             sgate=p(r.sgate), lrows=p(r.lbuf)))
+        e.set_inputs(dict(tokens=p(r.d_tokens), pos=p(r.d_pos), slot=p(r.d_slot), q_len=p(r.d_qlen),
+                          q_seq=p(r.d_qseq), block_table=p(r.d_block_table), max_blocks=r.max_blocks,
+                          bs=r.block_size, logits=p(r.logits), ld_logits=r.logits.shape[1],
+                          logit_idx=p(r.d_logit_idx)))
+        self.stages = dict(forward=C.ST_FORWARD, embed=C.ST_EMBED, run=C.ST_RUN, head=C.ST_HEAD)
+
+    def run(self, stage: str, layer: int, B: int, n_logits: int = 0, use_idx: bool = False, prefill: bool = False):
+        self.exe.step(self.stages[stage], layer, B, n_logits, use_idx, torch.cuda.current_stream().cuda_stream)
+
+
+class StackRunner(Runner):
+    def __init__(self, model_path: str, device: str | None = None, max_batch: int = 256, max_seqs: int = 4,
+                 ctx: int | None = None, block_size: int = 16, dtype: str = "bfloat16", kv_tokens: int = 0,
+                 use_graphs: bool | None = None, weights: StackWeights | None = None, cpu_backend: str | None = None):
+        """kv_tokens: tokens the block pool holds for all live sequences together (0: every slot at
+        `ctx`). ctx: longest sequence (default: the pool, or 4096). max_seqs: state slots = live sequences."""
+        t0 = time.perf_counter()
+        if device is None:
+            device = f"cuda:{torch.cuda.current_device()}" if torch.cuda.is_available() else "cpu"
+        self.device = dev = torch.device(device)
+        self.is_gpu = dev.type == "cuda"
+        if self.is_gpu:
+            self._sampler_module()  # fail loudly: no torch fallback on a GPU box
+        self.tp_rank, self.tp_size, self.tp_group, self.tp_ctrl, self.ar = 0, 1, None, None, None
+        self._closed = False
+        self.dtype = _DTYPES[dtype] if isinstance(dtype, str) else dtype
+        self.w = weights or StackWeights(model_path, dev, self.dtype)
+        cfg = self.cfg = self.w.cfg
+        self.runs = cfg.runs()
+        self.max_batch, self.max_seqs, self.block_size = max_batch, max_seqs, block_size
+        self.ctx = min(ctx or kv_tokens or 4096, cfg.ctx_len)
+        self.max_blocks = (self.ctx + block_size - 1) // block_size
+        n_blocks = self.pool_blocks(kv_tokens)
+        E, V, T = cfg.n_embd, cfg.n_vocab, self.dtype
+        f32 = dict(device=dev, dtype=torch.float32)
+        i32 = dict(device=dev, dtype=torch.int32)
+        tt = dict(device=dev, dtype=T)
+        # one cache per layer run
+        self.kc, self.vc, self.states = [], [], []
+        for li, _ps, _first in self.runs:
+            m = cfg.layers[li].mixer
+            if m.kind == MIX_ATTENTION:
+                self.kc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.dim, **tt))
+                self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
+                self.states.append(None)
+            else:
+                self.kc.append(None)
+                self.vc.append(None)
+                self.states.append(torch.zeros(max_seqs, m.heads, m.dim, m.vdim, **f32))
+        mlps = [s.mlp for s in cfg.layers if s.mlp is not None]
+        top = max([f.top for f in mlps], default=1)
+        self.resid = torch.zeros(max_batch, E, **f32)
+        self.x0 = torch.zeros(max_batch, E, **f32)          # the embedding output (re-enters at every pass)
+        self.hbuf = torch.zeros(max_batch, E, **tt)         # normed activations, the input projection's operand
+        self.catbuf = torch.zeros(max_batch, 2 * E, **tt)   # [x; x0], the pass-opening projection's operand
+        self.proj = torch.zeros(max_batch, max(L["n_in"] for L in self.w.layers), **f32)
+        self.abuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **tt)
+        self.hmid = torch.zeros(max_batch, max([f.top * f.ff + f.shared_ff for f in mlps], default=1), **tt)
+        self.ybuf = torch.zeros(max_batch, E, **f32)
+        self.eids = torch.zeros(max_batch, top, **i32)
+        self.ew = torch.zeros(max_batch, top, **f32)
+        self.sgate = torch.zeros(max_batch, **f32)
+        self.lbuf = torch.zeros(max_batch, E, **tt)
+        self.ext, self._ext_map, self._ext_next = None, {}, 0
+        self.mfma_bytes = self.lib_min = self.moe_lib = 0
+        self.w16 = self.mb_bufs = self.x8_bufs = None
+        self._alloc_step_state(V, n_blocks)
+        self.decode_group, self.graph_pair, self.steps_issued = 1, False, 0
+        self.ring_fence = 1 if os.environ.get("OMX_RING_FENCE", "0") == "1" else 0
+        self._defer_ok, self._decode_S, self._adv_next = False, 0, None
+        if self.is_gpu:
+            self.exe = StackExec(self)
+        else:
+            from ..ops.reference import TorchStackExecutor
+            self.exe = TorchStackExecutor(self)
+        self.cpu_backend = None if self.is_gpu else "torch"
+        if use_graphs is None:
+            use_graphs = self.is_gpu and os.environ.get("OMX_NO_GRAPH", "0") != "1"
+        self.use_graphs = use_graphs
+        self._alloc_host_side()
+        self.load_s = time.perf_counter() - t0
+
+    def _sampler_module(self):
+        from ..ops import stack_native
+        return stack_native()
+
+    # ------------------------------------------------------------------ step
+    def forward(self, B: int, n_logits: int, use_idx: bool = False, prefill: bool = False):
+        """One step over B rows; each row carries its own position, cache slot and sequence row, so rows of
+        several sequences (portions of prompts, single decode tokens) mix freely. Rows of one sequence are
+        contiguous and in position order."""
+        if self._closed:
+            raise RuntimeError("runner is closed")
+        self.exe.run("forward", 0, B, n_logits, use_idx, prefill)
+
+    def split_plan(self, B: int) -> tuple[int, int]:
+        return 1, 0
+
+    def _output_norm(self, h: torch.Tensor) -> torch.Tensor:
+        return torch.nn.functional.layer_norm(h, (h.shape[-1],), self.w.final_w, self.w.final_b, self.cfg.norm_eps)
+
+    # ------------------------------------------------------------------ sequences and state slots
+    def _clear_slot(self, row: int) -> None:
+        for st in self.states:
+            if st is not None:
+                st[row].zero_()
+
+    def new_sequence(self) -> int:
+        sid = super().new_sequence()
+        self._clear_slot(self.kv.seqs[sid].row)
+        return sid
+
+    def reusable_prefix(self, sid: int, n: int) -> int:
+        if not self.cfg.has_state:
+            return n
+        return n if n == self.kv.seqs[sid].length else 0
+
+    def _keep_prefix(self, sid: int, keep: int, history: list[int]) -> None:
+        s = self.kv.seqs[sid]
+        if self.cfg.has_state and keep != s.length:
+            if keep != 0:
+                raise RuntimeError(f"sequence {sid}: a recurrent state cannot be cut back from {s.length} to {keep}")
+            self._clear_slot(s.row)
+        super()._keep_prefix(sid, keep, history)
+
+    # ------------------------------------------------------------------ load-time warm-up
+    def warmup(self) -> None:
+        if not self.is_gpu:
+            return
+        V = self.cfg.n_vocab
+        for n in sorted({min(self.max_batch, 8), min(self.max_batch, 96)}):
+            sid = self.new_sequence()
+            try:
+                self.prefill(sid, [(i * 7919 + 3) % V for i in range(n)])
+            finally:
+                self.free_sequence(sid)
+        if self.use_graphs:
+            self._graph(1)
+        torch.cuda.synchronize()
+
+
+__all__ = ["StackRunner", "StackExec", "MIX_ATTENTION", "MIX_RETENTION"]

@@ -399,3 +399,85 @@ class DeviceWeights:
                 if isinstance(v, DevQMat):
                     n += v.nbytes
         return n
+
+
+# ---------------------------------------------------------------------------------------------------
+class StackWeights:
+    """Weights of a layer-list model (models/config.py StackConfig) from a folder with model.safetensors,
+    resident on `device` in `dtype` (bfloat16 as stored, or float32 for the exact mode). Every layer's
+    matrices that read the normed activations are stacked into ONE input projection `w_in`
+    (rows: q | k | v | [g] | router | shared gate scalar | shared gate | shared up), so a layer's step reads
+    its activations once; expert matrices are stacked [X][2F][E] (gate rows, then up rows) and [X][E][F]
+    so the kernels offset to the routed expert on the device. Norm weights, biases, decays and rotary
+    frequencies are float32."""
+
+    def __init__(self, path: str, device: str | torch.device = "cuda", dtype: torch.dtype = torch.bfloat16):
+        import os as _os
+
+        from ..models.config import MIX_RETENTION, load_stack_config
+        from .safetensors_io import SafetensorsFile
+        self.cfg = cfg = self.full_cfg = load_stack_config(path)
+        self.device, self.dtype = device, dtype
+        self.tp_rank, self.tp_size = 0, 1
+        st = SafetensorsFile(_os.path.join(path, "model.safetensors"))
+        E, V = cfg.n_embd, cfg.n_vocab
+
+        def get(name: str, shape: tuple) -> torch.Tensor:
+            if not st.has(name):
+                raise ValueError(f"{path}: tensor {name} is missing")
+            if st.shape(name) != tuple(shape):
+                raise ValueError(f"{path}: tensor {name} is {st.shape(name)}, expected {tuple(shape)}")
+            return st.tensor(name)
+
+        mat = lambda *ts: torch.cat([t.to(torch.float32) for t in ts], 0).to(dtype).contiguous().to(device)  # noqa: E731
+        vec = lambda t: t.to(torch.float32).reshape(-1).contiguous().to(device)  # noqa: E731
+        self.embed = mat(get("embed", (V, E)))
+        self.loop_in = mat(get("loop.in", (E, 2 * E))) if cfg.loop_times else None
+        self.layers = []
+        for i, spec in enumerate(cfg.layers):
+            m, f = spec.mixer, spec.mlp
+            p = f"l{i}."
+            L: dict = dict(norm_w=vec(get(p + "norm1", (E,))), norm_b=vec(get(p + "norm1.b", (E,))))
+            parts = [get(p + "mix.q", (m.n_q, E)), get(p + "mix.k", (m.n_k, E)), get(p + "mix.v", (m.n_v, E))]
+            off = dict(q=0, k=m.n_q, v=m.n_q + m.n_k)
+            n = m.n_q + m.n_k + m.n_v
+            if m.kind == MIX_RETENTION:
+                parts.append(get(p + "mix.g", (m.n_out, E)))
+                off["g"] = n
+                n += m.n_out
+                L["decay"] = torch.tensor(m.decay, dtype=torch.float32, device=device)
+                L["inv_freq"] = (torch.from_numpy(rope_inv_freq(m.rot_dims, m.rot_base)).to(device)
+                                 if m.rot_dims else None)
+            if f is not None:
+                X, F, Fs = f.experts, f.ff, f.shared_ff
+                parts.append(get(p + "mlp.router", (X, E)))
+                off["router"] = n
+                n += X
+                L["router_b"] = vec(get(p + "mlp.router.b", (X,)))
+                if Fs:
+                    parts += [get(p + "mlp.shared.sg", (1, E)), get(p + "mlp.shared.gate", (Fs, E)),
+                              get(p + "mlp.shared.up", (Fs, E))]
+                    off.update(sg=n, sgate=n + 1, sup=n + 1 + Fs)
+                    n += 1 + 2 * Fs
+                    L["sh_down"] = mat(get(p + "mlp.shared.down", (E, Fs)))
+                gu, dn = [], []
+                for e in range(X):
+                    q = f"{p}mlp.e{e}."
+                    gu += [get(q + "gate", (F, E)), get(q + "up", (F, E))]
+                    dn.append(get(q + "down", (E, F)))
+                L["w_gu"] = mat(*gu).view(X, 2 * F, E)
+                L["w_down"] = mat(*dn).view(X, E, F)
+            L["w_in"] = mat(*parts)
+            L["off"], L["n_in"] = off, n
+            L["w_o"] = mat(get(p + "mix.o", (E, m.n_out)))
+            self.layers.append(L)
+        self.final_w, self.final_b = vec(get("final.norm", (E,))), vec(get("final.norm.b", (E,)))
+        self.head = mat(get("head", (V, E)))
+        self.local = dict(E=E, V=V)
+
+    @property
+    def nbytes(self) -> int:
+        n = self.embed.numel() + self.head.numel() + (self.loop_in.numel() if self.loop_in is not None else 0)
+        for L in self.layers:
+            n += sum(v.numel() for v in L.values() if isinstance(v, torch.Tensor) and v.dtype == self.dtype)
+        return n * (2 if self.dtype == torch.bfloat16 else 4)

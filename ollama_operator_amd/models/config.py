@@ -236,3 +236,202 @@ PRESETS: dict[str, ModelConfig] = {
 
 def preset(name: str, **overrides) -> ModelConfig:
     return replace(PRESETS[name], **overrides)
+
+
+# ---------------------------------------------------------------------------------------------------
+# Layer-list models: a model given as a folder with config.json + model.safetensors whose config lists
+# heterogeneous layers (each with its own sequence mixer and feed-forward), optionally with a span of
+# layers that runs several times over the same weights. `STACK_ARCHS` maps config.json's "architecture"
+# to the reader that turns it into a StackConfig; the engine (engine/stack_runner.py) runs any StackConfig.
+
+MIX_ATTENTION = 0   # softmax attention over a paged key/value cache
+MIX_RETENTION = 1   # decayed linear attention with a per-sequence state matrix
+
+
+@dataclass
+class MixerSpec:
+    kind: int = MIX_ATTENTION
+    heads: int = 1
+    kv_heads: int = 1
+    dim: int = 64               # per-head query / key size
+    vdim: int = 64              # per-head value size
+    # attention
+    scale: float = 1.0          # score multiplier
+    softcap: float = 0.0        # score <- cap * tanh(score / cap); 0 = none
+    qtemp_coef: float = 0.0     # q *= 1 + coef * ln(floor((p + 1) / every) + 1); 0 = none
+    qtemp_every: int = 1
+    # retention
+    decay: tuple = ()           # per-head state decay
+    rot_dims: int = 0           # rotary dims per head (rotate-half pairing), 0 = none
+    rot_base: float = 10000.0
+
+    @property
+    def n_q(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def n_k(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def n_v(self) -> int:
+        return self.kv_heads * self.vdim
+
+    @property
+    def n_out(self) -> int:     # input width of the output projection
+        return self.heads * self.vdim
+
+
+@dataclass
+class MoESpec:
+    experts: int = 0
+    top: int = 0
+    ff: int = 0
+    shared_ff: int = 0          # 0 = no shared expert
+
+
+@dataclass
+class LayerSpec:
+    mixer: MixerSpec = field(default_factory=MixerSpec)
+    mlp: MoESpec | None = None
+
+
+@dataclass
+class StackConfig:
+    arch: str = "bizulix"
+    n_vocab: int = 0
+    n_embd: int = 0
+    layers: list = field(default_factory=list)   # [LayerSpec]
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 0         # 0 = no repeated span
+    norm_eps: float = 1e-5
+    residual_mult: float = 1.0
+    logit_softcap: float = 0.0
+    ctx_len: int = 1 << 20      # the design has no positional table: bounded by the cache pool only
+    bos_id: int = 0
+    eos_id: int = -1            # no tokenizer ships with these models: generation never stops on a token
+    name: str = ""
+    n_expert: int = 0           # (ModelConfig field the serving code reads; routing is per layer here)
+    n_expert_used: int = 0
+
+    @property
+    def n_layer(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list[tuple[int, int, bool]]:
+        """(layer, pass, opens a pass) in execution order: the repeated span [loop_start, loop_stop) runs
+        loop_times times in a row; every run has its own cache or state."""
+        L = len(self.layers)
+        if self.loop_times <= 0:
+            return [(i, 0, False) for i in range(L)]
+        a, b = self.loop_start, self.loop_stop
+        out = [(i, 0, False) for i in range(a)]
+        for p in range(self.loop_times):
+            out += [(i, p, i == a) for i in range(a, b)]
+        return out + [(i, 0, False) for i in range(b, L)]
+
+    @property
+    def has_state(self) -> bool:
+        """Some layer carries a recurrent state: a cached prefix cannot be cut back to an earlier length."""
+        return any(s.mixer.kind == MIX_RETENTION for s in self.layers)
+
+    def to_dict(self) -> dict:
+        return asdict(self)
+
+    # -- config.json of the Bizulix design
+    @classmethod
+    def from_bizulix(cls, c: dict) -> "StackConfig":
+        layers = []
+        for ent in c["layers"]:
+            m = ent["mixer"]
+            if ent["type"] == "attention":
+                qt = m.get("q_temp") or {}
+                mx = MixerSpec(kind=MIX_ATTENTION, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                               dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                               softcap=float(m.get("softcap") or 0.0), qtemp_coef=float(qt.get("coef", 0.0)),
+                               qtemp_every=int(qt.get("every", 1)))
+            elif ent["type"] == "retention":
+                rot = m.get("rot") or {}
+                mx = MixerSpec(kind=MIX_RETENTION, heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]),
+                               vdim=int(m.get("vdim", m["dim"])), decay=tuple(float(d) for d in m["decay"]),
+                               rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)))
+                if len(mx.decay) != mx.heads:
+                    raise UnsupportedArchitecture("retention: one decay per head expected")
+                if mx.rot_dims % 2 or mx.rot_dims > mx.dim:
+                    raise UnsupportedArchitecture("retention: rot.dims must be even and at most dim")
+            else:
+                raise UnsupportedArchitecture(f"unknown mixer type {ent['type']!r}")
+            if mx.heads % mx.kv_heads:
+                raise UnsupportedArchitecture("heads must be a multiple of kv_heads")
+            mlp = None
+            f = ent.get("mlp")
+            if f:
+                if f.get("kind", "moe") != "moe":
+                    raise UnsupportedArchitecture(f"unknown feed-forward kind {f.get('kind')!r}")
+                sh = f.get("shared") or {}
+                mlp = MoESpec(experts=int(f["router"]["experts"]), top=int(f["router"]["top"]),
+                              ff=int(f["expert"]["ff"]), shared_ff=int(sh.get("ff", 0)))
+                if not 0 < mlp.top <= mlp.experts:
+                    raise UnsupportedArchitecture("router: top must be in 1..experts")
+            layers.append(LayerSpec(mixer=mx, mlp=mlp))
+        loop = c.get("loop") or {}
+        cfg = cls(arch="bizulix", n_vocab=int(c["vocab"]), n_embd=int(c["width"]), layers=layers,
+                  loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+                  loop_times=int(loop.get("times", 0)) if loop else 0, norm_eps=float(c["norm"]["eps"]),
+                  residual_mult=float(c.get("residual_mult", 1.0)), logit_softcap=float(c.get("logit_softcap") or 0.0),
+                  name=str(c.get("name", "bizulix")))
+        if cfg.loop_times and not 0 <= cfg.loop_start < cfg.loop_stop <= len(layers):
+            raise UnsupportedArchitecture("loop: need 0 <= start < stop <= number of layers")
+        return cfg
+
+    def to_bizulix(self) -> dict:
+        """The config.json this configuration is read from (random-init fixtures, tests)."""
+        out = []
+        for s in self.layers:
+            m = s.mixer
+            if m.kind == MIX_ATTENTION:
+                d = dict(heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale)
+                if m.softcap:
+                    d["softcap"] = m.softcap
+                if m.qtemp_coef:
+                    d["q_temp"] = dict(coef=m.qtemp_coef, every=m.qtemp_every)
+                ent = dict(type="attention", mixer=d)
+            else:
+                d = dict(heads=m.heads, dim=m.dim, vdim=m.vdim, decay=list(m.decay))
+                if m.rot_dims:
+                    d["rot"] = dict(dims=m.rot_dims, base=m.rot_base)
+                ent = dict(type="retention", mixer=d)
+            f = s.mlp
+            ent["mlp"] = None if f is None else dict(
+                kind="moe", router=dict(experts=f.experts, top=f.top), expert=dict(ff=f.ff),
+                **({"shared": dict(ff=f.shared_ff)} if f.shared_ff else {}))
+            out.append(ent)
+        c = dict(architecture="Bizulix", vocab=self.n_vocab, width=self.n_embd, layers=out,
+                 norm=dict(eps=self.norm_eps), residual_mult=self.residual_mult)
+        if self.logit_softcap:
+            c["logit_softcap"] = self.logit_softcap
+        if self.loop_times:
+            c["loop"] = dict(start=self.loop_start, stop=self.loop_stop, times=self.loop_times)
+        return c
+
+
+STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix}
+
+
+def is_stack_model(path: str) -> bool:
+    """A model folder (config.json + model.safetensors) rather than a GGUF file."""
+    import os
+    return os.path.isdir(path) and os.path.exists(os.path.join(path, "config.json"))
+
+
+def load_stack_config(path: str) -> StackConfig:
+    import json
+    import os
+    with open(os.path.join(path, "config.json")) as f:
+        c = json.load(f)
+    arch = c.get("architecture")
+    if arch not in STACK_ARCHS:
+        raise UnsupportedArchitecture(
+            f"unsupported model architecture {arch!r} (config.json models: {', '.join(sorted(STACK_ARCHS))})")
+    return STACK_ARCHS[arch](c)

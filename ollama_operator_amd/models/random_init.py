@@ -51,3 +51,55 @@ def write_random_gguf(path: str, cfg: ModelConfig, ftype: FileType = FileType.MO
                 g, r, k, np.random.default_rng(s), std))
     w.write()
     return md
+
+
+def write_random_stack(path: str, cfg, seed: int = 0, std: float = 0.05) -> None:
+    """Random-init model folder (config.json + model.safetensors, bfloat16) of a layer-list model
+    (config.StackConfig, the Bizulix tensor names). Projections ~ N(0, std); norm weights near 1; router
+    matrices and biases wide enough that the top experts are not a close call."""
+    import json
+    import os
+
+    import torch
+
+    from ..engine.safetensors_io import write_safetensors
+    from .config import MIX_RETENTION
+    g = torch.Generator().manual_seed(seed)
+    E, V = cfg.n_embd, cfg.n_vocab
+    T: dict = {}
+
+    def rnd(name, shape, s=std, mean=0.0):
+        T[name] = (mean + s * torch.randn(*shape, generator=g)).to(torch.bfloat16)
+
+    rnd("embed", (V, E), 1.0)
+    if cfg.loop_times:
+        rnd("loop.in", (E, 2 * E), 0.7 / E ** 0.5)
+    for i, spec in enumerate(cfg.layers):
+        m, f, p = spec.mixer, spec.mlp, f"l{i}."
+        rnd(p + "norm1", (E,), 0.05, 1.0)
+        rnd(p + "norm1.b", (E,), 0.05)
+        rnd(p + "mix.q", (m.n_q, E), 1.0 / E ** 0.5)
+        rnd(p + "mix.k", (m.n_k, E), 1.0 / E ** 0.5)
+        rnd(p + "mix.v", (m.n_v, E), 1.0 / E ** 0.5)
+        if m.kind == MIX_RETENTION:
+            rnd(p + "mix.g", (m.n_out, E), 1.0 / E ** 0.5)
+        rnd(p + "mix.o", (E, m.n_out), 1.0 / m.n_out ** 0.5)
+        if f is not None:
+            for e in range(f.experts):
+                rnd(f"{p}mlp.e{e}.gate", (f.ff, E), 1.0 / E ** 0.5)
+                rnd(f"{p}mlp.e{e}.up", (f.ff, E), 1.0 / E ** 0.5)
+                rnd(f"{p}mlp.e{e}.down", (E, f.ff), 1.0 / f.ff ** 0.5)
+            rnd(p + "mlp.router", (f.experts, E), 2.0 / E ** 0.5)
+            rnd(p + "mlp.router.b", (f.experts,), 0.5)
+            if f.shared_ff:
+                rnd(p + "mlp.shared.gate", (f.shared_ff, E), 1.0 / E ** 0.5)
+                rnd(p + "mlp.shared.up", (f.shared_ff, E), 1.0 / E ** 0.5)
+                rnd(p + "mlp.shared.down", (E, f.shared_ff), 1.0 / f.shared_ff ** 0.5)
+                rnd(p + "mlp.shared.sg", (1, E), 1.0 / E ** 0.5)
+    rnd("final.norm", (E,), 0.05, 1.0)
+    rnd("final.norm.b", (E,), 0.05)
+    rnd("head", (V, E), 1.0 / E ** 0.5)
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as fh:
+        json.dump(cfg.to_bizulix(), fh, indent=1)
+    write_safetensors(os.path.join(path, "model.safetensors"), T)

@@ -27,6 +27,18 @@ def native():
     return _C
 
 
+def stack_native():
+    """The stack executor's module (`ollama_operator_amd/_stack`, csrc/stack: the kernels of layer-list
+    models, the sampler and the step feedback). It is its own small library, so a box that serves only
+    such a model builds it alone (`build_native.build_stack`)."""
+    try:
+        from .. import _stack  # type: ignore[attr-defined]
+    except ImportError as e:
+        raise RuntimeError(f"native extension ollama_operator_amd._stack is not built ({e}); "
+                           "run `python build_native.py --stack`") from None
+    return _stack
+
+
 def require_native_on_gpu() -> None:
     """Fail loudly when a GPU is present but the HIP extension is not."""
     if torch.cuda.is_available():

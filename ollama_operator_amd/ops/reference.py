@@ -195,3 +195,157 @@ class TorchExecutor:
 
 def np_to_i32(a) -> np.ndarray:
     return np.ascontiguousarray(a, dtype=np.int32)
+
+
+# ---------------------------------------------------------------------------------------------------
+# Torch twin of the stack executor (csrc/stack/stack_executor.cpp): the same buffers, the same places
+# where activations are rounded to the matrix dtype, float32 everywhere else. One function per kernel,
+# so a GPU test can compare kernel by kernel.
+
+def stack_matmul(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """a [M, K] and w [N, K] in the matrix dtype -> float32 [M, N] (products exact, float32 sums)."""
+    return a.float() @ w.float().T
+
+
+def stack_query_temperature(pos: torch.Tensor, coef: float, every: int) -> torch.Tensor:
+    return 1.0 + coef * torch.log(torch.floor((pos.float() + 1.0) / float(every)) + 1.0)
+
+
+def stack_attention(q, kc, vc, block_table, q_seq, q_len, bs, scale, softcap, groups):
+    """q [B, H, D] float32; kc [blocks, G, bs, D], vc [blocks, G, bs, Dv]; row b sees the first q_len[b]
+    keys of sequence row q_seq[b]. Returns float32 [B, H, Dv]."""
+    B, H, _ = q.shape
+    out = torch.empty(B, H, vc.shape[-1], dtype=torch.float32, device=q.device)
+    for b in range(B):
+        n = int(q_len[b])
+        t = torch.arange(n, device=q.device)
+        bt = block_table[int(q_seq[b])].long()
+        kk = kc[bt[t // bs], :, t % bs].float().repeat_interleave(groups, dim=1)  # [n, H, D]
+        vv = vc[bt[t // bs], :, t % bs].float().repeat_interleave(groups, dim=1)
+        s = torch.einsum("hd,thd->ht", q[b], kk) * scale
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
+        out[b] = torch.einsum("ht,thd->hd", torch.softmax(s, -1), vv)
+    return out
+
+
+def stack_rotate_half(x, pos, inv_freq):
+    """x [B, H, D] float32: dims i and i + R/2 (R = 2 * len(inv_freq)) rotate by pos * inv_freq[i]."""
+    half = inv_freq.numel()
+    ang = pos.float()[:, None] * inv_freq[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    u, v = x[..., :half], x[..., half:2 * half]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * half:]], -1)
+
+
+def stack_retention(q, k, v, state, q_seq, decay):
+    """q, k [B, H, D], v [B, H, Dv] float32, rows in sequence order; state [slots, H, D, Dv] is read and
+    advanced in place: S <- decay S + k v^T, o = S^T q. Returns float32 [B, H, Dv]."""
+    B = q.shape[0]
+    out = torch.empty_like(v)
+    for b in range(B):
+        S = state[int(q_seq[b])]
+        S.mul_(decay[:, None, None]).add_(k[b][:, :, None] * v[b][:, None, :])
+        out[b] = torch.einsum("hdv,hd->hv", S, q[b])
+    return out
+
+
+def stack_route(z: torch.Tensor, top: int):
+    """Router logits [B, X] -> (expert ids [B, top] by descending logit, softmax over the chosen logits)."""
+    val, idx = torch.topk(z, top, dim=-1)
+    return idx.to(torch.int32), torch.softmax(val, -1)
+
+
+class TorchStackExecutor:
+    def __init__(self, runner):
+        self.r = runner
+
+    def embed(self, B: int):
+        r = self.r
+        x = r.w.embed[r.d_tokens[:B].long()].float()
+        r.resid[:B] = x
+        r.x0[:B] = x
+
+    def layer_run(self, ri: int, B: int):
+        from ..models.config import MIX_ATTENTION
+        r = self.r
+        w, cfg, T = r.w, r.cfg, r.w.dtype
+        li, _ps, opens = r.runs[ri]
+        L, spec = w.layers[li], cfg.layers[li]
+        m, f, off = spec.mixer, spec.mlp, L["off"]
+        if opens:
+            r.catbuf[:B] = torch.cat([r.resid[:B], r.x0[:B]], 1).to(T)
+            r.resid[:B] = stack_matmul(r.catbuf[:B], w.loop_in)
+        x = r.resid[:B]
+        r.hbuf[:B] = F.layer_norm(x, (x.shape[-1],), L["norm_w"], L["norm_b"], cfg.norm_eps).to(T)
+        proj = stack_matmul(r.hbuf[:B], L["w_in"])
+        r.proj[:B, :proj.shape[1]] = proj
+        pos, qseq = r.d_pos[:B], r.d_qseq[:B]
+        q = proj[:, off["q"]:off["q"] + m.n_q].view(B, m.heads, m.dim)
+        k = proj[:, off["k"]:off["k"] + m.n_k].view(B, m.kv_heads, m.dim)
+        v = proj[:, off["v"]:off["v"] + m.n_v].view(B, m.kv_heads, m.vdim)
+        if m.kind == MIX_ATTENTION:
+            if m.qtemp_coef:
+                q = q * stack_query_temperature(pos, m.qtemp_coef, m.qtemp_every)[:, None, None]
+            slot = r.d_slot[:B].long()
+            blk, o = slot // r.block_size, slot % r.block_size
+            r.kc[ri][blk, :, o] = k.to(T)
+            r.vc[ri][blk, :, o] = v.to(T)
+            a = stack_attention(q, r.kc[ri], r.vc[ri], r.d_block_table, qseq, r.d_qlen[:B], r.block_size, m.scale,
+                                m.softcap, m.heads // m.kv_heads)
+        else:
+            if m.rot_dims:
+                q = stack_rotate_half(q, pos, L["inv_freq"])
+                k = stack_rotate_half(k, pos, L["inv_freq"])
+            k = k * float(m.dim) ** -0.5
+            o = stack_retention(q, k, v, r.states[ri], qseq, L["decay"])
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + cfg.norm_eps)
+            g = proj[:, off["g"]:off["g"] + m.n_out].view(B, m.heads, m.vdim)
+            a = o * F.silu(g)
+        r.abuf[:B, :m.n_out] = a.reshape(B, m.n_out).to(T)
+        y = stack_matmul(r.abuf[:B, :m.n_out], L["w_o"])
+        if f is not None:
+            z = proj[:, off["router"]:off["router"] + f.experts] + L["router_b"]
+            ids, wt = stack_route(z, f.top)
+            r.eids[:B, :f.top], r.ew[:B, :f.top] = ids, wt
+            h = r.hbuf[:B]
+            ff = torch.zeros_like(y)
+            for b in range(B):
+                for j in range(f.top):
+                    e = int(ids[b, j])
+                    gu = stack_matmul(h[b:b + 1], L["w_gu"][e])[0]
+                    mid = (F.silu(gu[:f.ff]) * gu[f.ff:]).to(T)
+                    ff[b] += wt[b, j] * stack_matmul(mid[None], L["w_down"][e])[0]
+            if f.shared_ff:
+                Fs = f.shared_ff
+                mid = (F.silu(proj[:, off["sgate"]:off["sgate"] + Fs]) * proj[:, off["sup"]:off["sup"] + Fs]).to(T)
+                ff += torch.sigmoid(proj[:, off["sg"]:off["sg"] + 1]) * stack_matmul(mid, L["sh_down"])
+            y = y + ff
+        r.resid[:B] = x + cfg.residual_mult * y
+
+    def head(self, n_logits: int, use_idx: bool):
+        r = self.r
+        if n_logits <= 0:
+            return
+        w, cfg = r.w, r.cfg
+        x = r.resid[r.d_logit_idx[:n_logits].long()] if use_idx else r.resid[:n_logits]
+        r.lbuf[:n_logits] = F.layer_norm(x, (x.shape[-1],), w.final_w, w.final_b, cfg.norm_eps).to(w.dtype)
+        z = stack_matmul(r.lbuf[:n_logits], w.head)
+        if cfg.logit_softcap:
+            z = cfg.logit_softcap * torch.tanh(z / cfg.logit_softcap)
+        r.logits[:n_logits, :z.shape[1]] = z
+
+    def run(self, stage: str, layer: int, B: int, n_logits: int = 0, use_idx: bool = False, prefill: bool = False):
+        if stage == "embed":
+            self.embed(B)
+        elif stage == "run":
+            self.layer_run(layer, B)
+        elif stage == "head":
+            self.head(n_logits, use_idx)
+        elif stage == "forward":
+            self.embed(B)
+            for ri in range(len(self.r.runs)):
+                self.layer_run(ri, B)
+            self.head(n_logits, use_idx)
+        else:
+            raise ValueError(stage)
