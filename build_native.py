@@ -20,6 +20,7 @@ import sysconfig
 ROOT = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(ROOT, "csrc")
 CPU_SRC = os.path.join(CSRC, "cpu")
+STACK_SRC = os.path.join(CSRC, "stack")
 BUILD = os.path.join(ROOT, "build", "native")
 ARCH = os.environ.get("OMX_ARCH", "gfx950")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -74,7 +75,8 @@ def build(jobs: int | None = None, clean: bool = False, verbose: bool = False, d
             os.remove(f)
     srcs = sorted(s for s in glob.glob(os.path.join(CSRC, "**", "*.hip"), recursive=True) +
                   glob.glob(os.path.join(CSRC, "**", "*.cpp"), recursive=True)
-                  if not s.startswith(CPU_SRC + os.sep))  # the CPU backend is its own module (build_cpu)
+                  if not s.startswith(CPU_SRC + os.sep)  # the CPU backend is its own module (build_cpu)
+                  and not s.startswith(STACK_SRC + os.sep))  # and so is the stack executor (build_stack)
     hdr_mtime = max((os.path.getmtime(h) for h in _headers()), default=0.0)
     py_inc = sysconfig.get_paths()["include"]
     if sources is not None:
@@ -138,6 +140,70 @@ def build(jobs: int | None = None, clean: bool = False, verbose: bool = False, d
     return out
 
 
+def stack_target_path() -> str:
+    return os.path.join(ROOT, "ollama_operator_amd", "_stack" + _ext_suffix())
+
+
+# HIP device code is compiled without packed-float32 instructions (the compiler otherwise forms them from
+# ordinary float code)
+NO_PK_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_stack(verbose: bool = False, force: bool = False) -> str:
+    """`ollama_operator_amd/_stack*.so`: the kernels and step executor of layer-list models (csrc/stack) with
+    the on-device sampler (csrc/kernels/sampling.hip). Its own small library: a checkout that serves only
+    such a model compiles these few files (about a minute), not the quantised-GEMV families of `_C`."""
+    import pybind11
+    build_dir = os.path.join(ROOT, "build", "stack")
+    os.makedirs(build_dir, exist_ok=True)
+    srcs = sorted(glob.glob(os.path.join(STACK_SRC, "*.hip")) + glob.glob(os.path.join(STACK_SRC, "*.cpp")))
+    srcs.append(os.path.join(CSRC, "kernels", "sampling.hip"))
+    hdr_mtime = max((os.path.getmtime(h) for h in _headers()), default=0.0)
+    common = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-I", CSRC, "-I", pybind11.get_include(),
+              "-I", sysconfig.get_paths()["include"], "-Wno-unused-result"]
+    todo, objs = [], []
+    for s in srcs:
+        obj = os.path.join(build_dir, os.path.relpath(s, CSRC).replace(os.sep, "_") + ".o")
+        objs.append(obj)
+        if force or _needs(obj, s, hdr_mtime):
+            if s.endswith(".hip"):
+                cmd = [HIPCC, *common, *NO_PK_F32, "-c", s, "-o", obj]
+            else:
+                cmd = [HIPCC, *common, "-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-c", s, "-o", obj,
+                       "-fvisibility=hidden"]
+            todo.append((s, cmd))
+
+    def run(item):
+        s, cmd = item
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        return s, r.returncode, r.stdout + r.stderr, " ".join(cmd)
+
+    failed = []
+    if todo:
+        with cf.ThreadPoolExecutor(max_workers=min(8, len(todo))) as ex:
+            for s, rc, out, cmd in ex.map(run, todo):
+                if rc != 0:
+                    failed.append((s, out, cmd))
+                elif verbose:
+                    print("compiled", os.path.relpath(s, ROOT))
+    if failed:
+        for s, out, cmd in failed:
+            sys.stderr.write(f"--- {s}\n{cmd}\n{out}\n")
+        raise RuntimeError(f"stack module build failed ({len(failed)} translation units)")
+    out = stack_target_path()
+    if not os.path.exists(out) or todo or any(os.path.getmtime(o) > os.path.getmtime(out) for o in objs):
+        tmp = out + ".tmp"
+        link = [HIPCC, "-shared", f"--offload-arch={ARCH}", "-o", tmp, *objs, "-lpthread"]
+        tl = _torch_lib()
+        if tl:
+            link += [f"-L{tl}", f"-Wl,-rpath,{tl}"]
+        r = subprocess.run(link, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + " ".join(link) + "\n" + r.stdout + r.stderr)
+        os.replace(tmp, out)
+    return out
+
+
 def cpu_target_path() -> str:
     return os.path.join(ROOT, "ollama_operator_amd", "_cpu" + _ext_suffix())
 
@@ -169,9 +235,15 @@ if __name__ == "__main__":
     ap.add_argument("--clean", action="store_true")
     ap.add_argument("--jobs", type=int, default=None)
     ap.add_argument("--cpu-only", action="store_true", help="build only the CPU backend module")
+    ap.add_argument("--stack", action="store_true", help="build only the stack executor's module")
     ap.add_argument("--debug", action="store_true",
                     help="kernels with in-kernel bounds assertions (OMX_KASSERT), -O1 -g, into build/debug")
     a = ap.parse_args()
+    if a.stack:
+        print(build_stack(verbose=True))
+        sys.exit(0)
+    if not a.debug:
+        print(build_stack(verbose=True))
     if not a.debug:
         print(build_cpu(verbose=True))
     if not a.cpu_only:

@@ -10,6 +10,7 @@
 #include <memory>
 #include <stdexcept>
 
+#include "bind_sampling.h"
 #include "gguf/gguf.h"
 #include "kernels/ops.h"
 #include "runtime/executor.h"
@@ -374,59 +375,7 @@ PYBIND11_MODULE(_C, m) {
     widen_q6k(q, Pp<void>(out), S(stream));
   });
   // host-mapped pinned buffer: (host pointer, device pointer); kernels store tokens into it directly
-  m.def("host_alloc_mapped", [](size_t bytes) {
-    void* h = nullptr;
-    void* d = nullptr;
-    if (hipHostMalloc(&h, bytes, hipHostMallocMapped) != hipSuccess || !h)
-      throw std::runtime_error("hipHostMalloc(mapped) failed");
-    if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess || !d) {
-      (void)hipHostFree(h);
-      throw std::runtime_error("hipHostGetDevicePointer failed");
-    }
-    std::memset(h, 0, bytes);
-    return py::make_tuple((uintptr_t)h, (uintptr_t)d);
-  });
-  m.def("host_free_mapped", [](uintptr_t h) {
-    if (h) (void)hipHostFree((void*)h);
-  });
-  m.def("sample", [](py::dict d, uintptr_t stream) {
-    SampleParams P{};
-    P.logits = Pp<const float>(d["logits"].cast<uintptr_t>());
-    P.B = d["B"].cast<int>();
-    P.V = d["V"].cast<int>();
-    P.ld = d["ld"].cast<int>();
-    P.temperature = Pp<const float>(d["temperature"].cast<uintptr_t>());
-    P.top_k = Pp<const int>(d["top_k"].cast<uintptr_t>());
-    P.top_p = Pp<const float>(d["top_p"].cast<uintptr_t>());
-    P.min_p = Pp<const float>(d["min_p"].cast<uintptr_t>());
-    P.repeat_penalty = Pp<const float>(d["repeat_penalty"].cast<uintptr_t>());
-    P.presence_penalty = Pp<const float>(d["presence_penalty"].cast<uintptr_t>());
-    P.frequency_penalty = Pp<const float>(d["frequency_penalty"].cast<uintptr_t>());
-    P.history = Pp<int>(d["history"].cast<uintptr_t>());
-    P.hist_count = Pp<int>(d["hist_count"].cast<uintptr_t>());
-    P.hist_cap = d["hist_cap"].cast<int>();
-    P.repeat_last_n = Pp<const int>(d["repeat_last_n"].cast<uintptr_t>());
-    P.seed = Pp<const unsigned long long>(d["seed"].cast<uintptr_t>());
-    P.step = Pp<int>(d["step"].cast<uintptr_t>());
-    P.out = Pp<int>(d["out"].cast<uintptr_t>());
-    P.out_logprob = Pp<float>(d.contains("out_logprob") ? d["out_logprob"].cast<uintptr_t>() : 0);
-    P.ws = Pp<float>(d.contains("ws") ? d["ws"].cast<uintptr_t>() : 0);
-    P.counters = Pp<int>(d.contains("counters") ? d["counters"].cast<uintptr_t>() : 0);
-    P.err = Pp<int>(d.contains("err") ? d["err"].cast<uintptr_t>() : 0);
-    if (d.contains("fb_step")) {
-      P.fb_step = Pp<int>(d["fb_step"].cast<uintptr_t>());
-      P.fb_ld = d["fb_ld"].cast<int>();
-      P.fb_block_table = Pp<const int>(d["fb_block_table"].cast<uintptr_t>());
-      P.fb_max_blocks = d["fb_max_blocks"].cast<int>();
-      P.fb_bs = d["fb_bs"].cast<int>();
-      P.fb_host_ring = Pp<int>(d.contains("fb_host_ring") ? d["fb_host_ring"].cast<uintptr_t>() : 0);
-      P.fb_ring = d.contains("fb_ring") ? d["fb_ring"].cast<int>() : 0;
-      P.fb_sysfence = d.contains("fb_sysfence") ? d["fb_sysfence"].cast<int>() : 1;
-      if (P.B > P.fb_ld || P.fb_bs <= 0 || P.fb_max_blocks <= 0) throw std::runtime_error("sample: bad feedback args");
-      if (P.fb_host_ring && P.fb_ring <= 0) throw std::runtime_error("sample: bad feedback ring");
-    }
-    sample(P, S(stream));
-  });
+  bind_sampling(m);
 
   // ------------------------------------------------------------------ executor
   py::class_<Executor>(m, "Executor")

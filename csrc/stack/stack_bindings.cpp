@@ -1,0 +1,174 @@
+// Python bindings of the stack executor's module (`ollama_operator_amd/_stack`): the executor, the matrix
+// product on its own (kernel tests), and the sampler shared with the main module. Torch-header-free:
+// device pointers and streams cross as integers.
+#include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <stdexcept>
+
+#include "../bind_sampling.h"
+#include "stack_executor.h"
+
+namespace py = pybind11;
+using namespace omx::stack;
+
+template <class T>
+static inline T* Pp(uintptr_t p) { return reinterpret_cast<T*>(p); }
+static inline hipStream_t S(uintptr_t s) { return reinterpret_cast<hipStream_t>(s); }
+static uintptr_t ptr(const py::dict& d, const char* k) { return d.contains(k) ? d[k].cast<uintptr_t>() : 0; }
+static int geti(const py::dict& d, const char* k, int dflt = 0) { return d.contains(k) ? d[k].cast<int>() : dflt; }
+static float getf(const py::dict& d, const char* k, float dflt = 0.f) { return d.contains(k) ? d[k].cast<float>() : dflt; }
+
+enum { ST_FORWARD = 0, ST_EMBED = 1, ST_RUN = 2, ST_HEAD = 3 };
+
+PYBIND11_MODULE(_stack, m) {
+  m.doc() = "gfx950 kernels and step executor of layer-list models";
+  omx::bind_sampling(m);
+  m.attr("ST_FORWARD") = (int)ST_FORWARD;
+  m.attr("ST_EMBED") = (int)ST_EMBED;
+  m.attr("ST_RUN") = (int)ST_RUN;
+  m.attr("ST_HEAD") = (int)ST_HEAD;
+  m.def("gemm", [](py::dict d, uintptr_t stream) {
+    GemmParams P{};
+    P.A = Pp<const void>(ptr(d, "A"));
+    P.lda = geti(d, "lda");
+    P.W = Pp<const void>(ptr(d, "W"));
+    P.M = geti(d, "M");
+    P.N = geti(d, "N");
+    P.K = geti(d, "K");
+    P.C = Pp<float>(ptr(d, "C"));
+    P.ldc = geti(d, "ldc");
+    P.epi = geti(d, "epi");
+    P.mult = getf(d, "mult", 1.f);
+    P.add = Pp<const float>(ptr(d, "add"));
+    P.cap = getf(d, "cap");
+    P.f32 = geti(d, "f32");
+    gemm(P, S(stream));
+  });
+  m.def("gemm_path", &gemm_path);
+  m.def("set_gemm_mfma", &set_gemm_mfma);
+  m.def("retention_supported", &retention_supported);
+
+  py::class_<StackExecutor>(m, "Executor")
+      .def(py::init<>())
+      .def("configure", [](StackExecutor& e, py::dict c) {
+        e.cfg.E = geti(c, "E");
+        e.cfg.V = geti(c, "V");
+        e.cfg.eps = getf(c, "eps", 1e-5f);
+        e.cfg.residual_mult = getf(c, "residual_mult", 1.f);
+        e.cfg.logit_softcap = getf(c, "logit_softcap");
+        e.cfg.f32 = geti(c, "f32");
+        e.cfg.max_B = geti(c, "max_B");
+        e.cfg.max_seqs = geti(c, "max_seqs");
+      })
+      .def("set_globals", [](StackExecutor& e, py::dict d) {
+        e.embed_w = Pp<const void>(ptr(d, "embed"));
+        e.loop_in = Pp<const void>(ptr(d, "loop_in"));
+        e.final_w = Pp<const float>(ptr(d, "final_w"));
+        e.final_b = Pp<const float>(ptr(d, "final_b"));
+        e.head_w = Pp<const void>(ptr(d, "head"));
+      })
+      .def("set_layer", [](StackExecutor& e, int i, py::dict d) {
+        if (i < 0) throw std::runtime_error("bad layer index");
+        if ((int)e.layers.size() <= i) e.layers.resize(i + 1);
+        LayerDesc& L = e.layers[i];
+        L = LayerDesc{};
+        L.kind = geti(d, "kind");
+        L.heads = geti(d, "heads");
+        L.kv_heads = geti(d, "kv_heads");
+        L.dim = geti(d, "dim");
+        L.vdim = geti(d, "vdim");
+        L.scale = getf(d, "scale", 1.f);
+        L.softcap = getf(d, "softcap");
+        L.qtemp_coef = getf(d, "qtemp_coef");
+        L.qtemp_every = geti(d, "qtemp_every", 1);
+        L.rot_dims = geti(d, "rot_dims");
+        L.n_in = geti(d, "n_in");
+        L.off_q = geti(d, "off_q");
+        L.off_k = geti(d, "off_k");
+        L.off_v = geti(d, "off_v");
+        L.off_g = geti(d, "off_g");
+        L.off_router = geti(d, "off_router");
+        L.off_sg = geti(d, "off_sg");
+        L.off_sgate = geti(d, "off_sgate");
+        L.off_sup = geti(d, "off_sup");
+        L.norm_w = Pp<const float>(ptr(d, "norm_w"));
+        L.norm_b = Pp<const float>(ptr(d, "norm_b"));
+        L.w_in = Pp<const void>(ptr(d, "w_in"));
+        L.w_o = Pp<const void>(ptr(d, "w_o"));
+        L.decay = Pp<const float>(ptr(d, "decay"));
+        L.inv_freq = Pp<const float>(ptr(d, "inv_freq"));
+        L.experts = geti(d, "experts");
+        L.top = geti(d, "top");
+        L.ff = geti(d, "ff");
+        L.shared_ff = geti(d, "shared_ff");
+        L.router_b = Pp<const float>(ptr(d, "router_b"));
+        L.w_gu = Pp<const void>(ptr(d, "w_gu"));
+        L.w_down = Pp<const void>(ptr(d, "w_down"));
+        L.sh_down = Pp<const void>(ptr(d, "sh_down"));
+        if (L.qtemp_every <= 0) throw std::runtime_error("q_temp.every must be positive");
+      })
+      .def("set_runs", [](StackExecutor& e, std::vector<py::dict> runs) {
+        e.runs.clear();
+        for (auto& d : runs) {
+          RunDesc r;
+          r.layer = geti(d, "layer");
+          r.opens_pass = geti(d, "opens_pass");
+          r.kc = Pp<void>(ptr(d, "kc"));
+          r.vc = Pp<void>(ptr(d, "vc"));
+          r.state = Pp<float>(ptr(d, "state"));
+          e.runs.push_back(r);
+        }
+      })
+      .def("set_workspace", [](StackExecutor& e, py::dict d) {
+        StackWorkspace& w = e.ws;
+        w.resid = Pp<float>(ptr(d, "resid"));
+        w.x0 = Pp<float>(ptr(d, "x0"));
+        w.h = Pp<void>(ptr(d, "h"));
+        w.cat = Pp<void>(ptr(d, "cat"));
+        w.proj = Pp<float>(ptr(d, "proj"));
+        w.ld_proj = geti(d, "ld_proj");
+        w.a = Pp<void>(ptr(d, "a"));
+        w.ld_a = geti(d, "ld_a");
+        w.hmid = Pp<void>(ptr(d, "hmid"));
+        w.ld_hmid = geti(d, "ld_hmid");
+        w.y = Pp<float>(ptr(d, "y"));
+        w.eids = Pp<int>(ptr(d, "eids"));
+        w.ew = Pp<float>(ptr(d, "ew"));
+        w.ld_top = geti(d, "ld_top");
+        w.sgate = Pp<float>(ptr(d, "sgate"));
+        w.lrows = Pp<void>(ptr(d, "lrows"));
+      })
+      .def("set_inputs", [](StackExecutor& e, py::dict d) {
+        StackInputs& in = e.in;
+        in.tokens = Pp<const int>(ptr(d, "tokens"));
+        in.pos = Pp<const int>(ptr(d, "pos"));
+        in.slot = Pp<const int>(ptr(d, "slot"));
+        in.q_len = Pp<const int>(ptr(d, "q_len"));
+        in.q_seq = Pp<const int>(ptr(d, "q_seq"));
+        in.block_table = Pp<const int>(ptr(d, "block_table"));
+        in.max_blocks = geti(d, "max_blocks");
+        in.bs = geti(d, "bs", 16);
+        in.logits = Pp<float>(ptr(d, "logits"));
+        in.ld_logits = geti(d, "ld_logits");
+        in.logit_idx = Pp<const int>(ptr(d, "logit_idx"));
+        if (in.bs <= 0 || in.max_blocks <= 0) throw std::runtime_error("bad block geometry");
+        e.validate();
+      })
+      .def("step", [](StackExecutor& e, int stage, int idx, int B, int n_logits, bool use_idx, uintptr_t stream) {
+        if (B <= 0 || B > e.cfg.max_B || n_logits < 0 || n_logits > e.cfg.max_B)
+          throw std::runtime_error("stack executor: rows outside 1..max_B");
+        if (use_idx && !e.in.logit_idx) throw std::runtime_error("stack executor: no logit index bound");
+        hipStream_t s = S(stream);
+        switch (stage) {
+          case ST_FORWARD: e.forward(B, n_logits, use_idx, s); break;
+          case ST_EMBED: e.embed(B, s); break;
+          case ST_RUN:
+            if (idx < 0 || idx >= (int)e.runs.size()) throw std::runtime_error("stack executor: bad run index");
+            e.layer_run(idx, B, s);
+            break;
+          case ST_HEAD: e.head(n_logits, use_idx, s); break;
+          default: throw std::runtime_error("stack executor: unknown stage");
+        }
+      });
+}

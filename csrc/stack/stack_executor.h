@@ -1,0 +1,102 @@
+// Step executor of layer-list models: the launch sequence of one step over B rows (any mix of prompt
+// portions and single decode tokens; rows of a sequence contiguous and in position order). Python owns
+// the device memory and hands raw pointers in; the executor only enqueues kernels on a stream, so a whole
+// step is capturable into one hipGraph.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <vector>
+
+#include "stack_ops.h"
+
+namespace omx {
+namespace stack {
+
+struct StackConfig {
+  int E = 0, V = 0;
+  float eps = 1e-5f, residual_mult = 1.f, logit_softcap = 0.f;
+  int f32 = 0;
+  int max_B = 0, max_seqs = 0;
+};
+
+struct LayerDesc {
+  int kind = 0;  // 0 attention, 1 retention
+  int heads = 0, kv_heads = 0, dim = 0, vdim = 0;
+  float scale = 1.f, softcap = 0.f, qtemp_coef = 0.f;
+  int qtemp_every = 1, rot_dims = 0;
+  int n_in = 0, off_q = 0, off_k = 0, off_v = 0, off_g = 0, off_router = 0, off_sg = 0, off_sgate = 0, off_sup = 0;
+  const float* norm_w = nullptr;
+  const float* norm_b = nullptr;
+  const void* w_in = nullptr;   // [n_in][E]
+  const void* w_o = nullptr;    // [E][heads * vdim]
+  const float* decay = nullptr;
+  const float* inv_freq = nullptr;
+  int experts = 0, top = 0, ff = 0, shared_ff = 0;  // experts == 0: no feed-forward
+  const float* router_b = nullptr;
+  const void* w_gu = nullptr;
+  const void* w_down = nullptr;
+  const void* sh_down = nullptr;
+};
+
+struct RunDesc {   // one execution of a layer: its own cache
+  int layer = 0;
+  int opens_pass = 0;  // x <- W_in [x; x0] first
+  void* kc = nullptr;
+  void* vc = nullptr;
+  float* state = nullptr;
+};
+
+struct StackWorkspace {
+  float* resid = nullptr;  // [max_B][E]
+  float* x0 = nullptr;     // [max_B][E]
+  void* h = nullptr;       // [max_B][E] matrix dtype
+  void* cat = nullptr;     // [max_B][2E] matrix dtype
+  float* proj = nullptr;   // [max_B][ld_proj]
+  int ld_proj = 0;
+  void* a = nullptr;       // [max_B][ld_a] matrix dtype (mixer output before the output projection)
+  int ld_a = 0;
+  void* hmid = nullptr;
+  int ld_hmid = 0;
+  float* y = nullptr;      // [max_B][E] feed-forward output
+  int* eids = nullptr;
+  float* ew = nullptr;
+  int ld_top = 0;
+  float* sgate = nullptr;
+  void* lrows = nullptr;   // [max_B][E] matrix dtype: normed rows for the head
+};
+
+struct StackInputs {
+  const int* tokens = nullptr;
+  const int* pos = nullptr;
+  const int* slot = nullptr;
+  const int* q_len = nullptr;
+  const int* q_seq = nullptr;
+  const int* block_table = nullptr;
+  int max_blocks = 0, bs = 16;
+  float* logits = nullptr;
+  int ld_logits = 0;
+  const int* logit_idx = nullptr;
+};
+
+class StackExecutor {
+ public:
+  StackConfig cfg;
+  std::vector<LayerDesc> layers;
+  std::vector<RunDesc> runs;
+  const void* embed_w = nullptr;
+  const void* loop_in = nullptr;
+  const float* final_w = nullptr;
+  const float* final_b = nullptr;
+  const void* head_w = nullptr;
+  StackWorkspace ws;
+  StackInputs in;
+
+  void validate() const;  // throws when a size does not fit the kernels or a pointer is missing
+  void embed(int B, hipStream_t s);
+  void layer_run(int ri, int B, hipStream_t s);
+  void head(int n_logits, bool use_idx, hipStream_t s);
+  void forward(int B, int n_logits, bool use_idx, hipStream_t s);
+};
+
+}  // namespace stack
+}  // namespace omx

@@ -1,0 +1,716 @@
+// gfx950 kernels of layer-list models (interface and operand layouts: stack_ops.h). Every kernel is
+// instantiated for bfloat16 and float32 matrices; norms, scores, softmax weights, router logits, the
+// retention state and the residual stream are float32 in both. Wave = 64 lanes.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <stdexcept>
+#include <string>
+
+#include "stack_ops.h"
+
+namespace omx {
+namespace stack {
+
+struct bf16 {
+  uint16_t v;
+};
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+// round to nearest even, as torch's float -> bfloat16 conversion
+__device__ __forceinline__ uint16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float ld(const float* p) { return *p; }
+__device__ __forceinline__ float ld(const bf16* p) { return bf2f(p->v); }
+__device__ __forceinline__ void st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st(bf16* p, float v) { p->v = f2bf(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+// sum over a block of 256 threads; every thread gets the result. red: 4 floats of LDS
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+__device__ __forceinline__ float silu(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float sigmoidf(float z) { return 1.f / (1.f + expf(-z)); }
+
+static void check(bool ok, const char* what) {
+  if (!ok) throw std::runtime_error(std::string("stack kernels: ") + what);
+}
+static void launched(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) throw std::runtime_error(std::string("stack kernels: ") + what + ": " + hipGetErrorString(e));
+}
+
+// ------------------------------------------------------------------------------------------------
+// dot product of two rows over a wave: 16-byte loads when both rows allow it
+template <typename T>
+__device__ __forceinline__ float wave_dot(const T* __restrict__ w, const T* __restrict__ x, int K, int lane, bool vec);
+template <>
+__device__ __forceinline__ float wave_dot<bf16>(const bf16* __restrict__ w, const bf16* __restrict__ x, int K, int lane,
+                                                bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int k = lane * 8; k < K; k += 512) {
+      const u32x4 a = *(const u32x4*)(w + k), b = *(const u32x4*)(x + k);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc += __uint_as_float(a[i] << 16) * __uint_as_float(b[i] << 16);
+        acc += __uint_as_float(a[i] & 0xffff0000u) * __uint_as_float(b[i] & 0xffff0000u);
+      }
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) acc += ld(w + k) * ld(x + k);
+  }
+  return wave_sum(acc);
+}
+template <>
+__device__ __forceinline__ float wave_dot<float>(const float* __restrict__ w, const float* __restrict__ x, int K, int lane,
+                                                 bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int k = lane * 4; k < K; k += 256) {
+      const f32x4 a = *(const f32x4*)(w + k), b = *(const f32x4*)(x + k);
+      acc += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) acc += w[k] * x[k];
+  }
+  return wave_sum(acc);
+}
+template <typename T>
+static inline bool vec_ok(const void* p, long long ld_elems, int K) {
+  const int per = 16 / (int)sizeof(T);
+  return K % per == 0 && ld_elems % per == 0 && ((uintptr_t)p & 15) == 0;
+}
+
+// ------------------------------------------------------------------------------------------------ epilogue
+struct Epi {
+  int mode;
+  float* C;
+  int ldc;
+  float mult;
+  const float* add;
+  float cap;
+};
+__device__ __forceinline__ void epi_store(const Epi& e, int m, int n, float acc) {
+  float* c = e.C + (long long)m * e.ldc + n;
+  if (e.mode == EPI_RESID) {
+    const float extra = e.add ? e.add[(long long)m * e.ldc + n] : 0.f;
+    *c = *c + e.mult * (acc + extra);
+  } else if (e.mode == EPI_SOFTCAP && e.cap != 0.f) {
+    *c = e.cap * tanhf(acc / e.cap);
+  } else {
+    *c = acc;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ GEMV (M <= 8)
+// one wave per weight row; the row is read once and meets every activation row
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_rows_kernel(const T* __restrict__ A, int lda, const T* __restrict__ W, int M,
+                                                        int N, int K, Epi e, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const T* w = W + (long long)n * K;
+  for (int m = 0; m < M; ++m) {
+    const float acc = wave_dot<T>(w, A + (long long)m * lda, K, lane, vec != 0);
+    if (lane == 0) epi_store(e, m, n, acc);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ FMA tile GEMM
+// 64 x 64 output tile per block, K in steps of 16 through LDS, 4 x 4 outputs per thread; true float32
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_fma_kernel(const T* __restrict__ A, int lda, const T* __restrict__ W, int M,
+                                                       int N, int K, Epi e) {
+  __shared__ float As[16][68];
+  __shared__ float Ws[16][68];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = tid & 15, ty = tid >> 4;
+  float acc[4][4] = {};
+  const int lr = tid >> 2, lk = (tid & 3) * 4;  // this thread stages row lr, k lk .. lk + 3 of both tiles
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + lk + j;
+      As[lk + j][lr] = (m0 + lr < M && k < K) ? ld(A + (long long)(m0 + lr) * lda + k) : 0.f;
+      Ws[lk + j][lr] = (n0 + lr < N && k < K) ? ld(W + (long long)(n0 + lr) * K + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Ws[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+      if (m < M && n < N) epi_store(e, m, n, acc[i][j]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ MFMA tile GEMM
+// bfloat16: (32 TM) x (32 TN) output tile per block of 4 waves (2 x 2), each wave TM x TN fragments of
+// v_mfma_f32_32x32x16_bf16; K in steps of 32 through LDS (rows padded to 40 elements so the 16-byte
+// fragment reads of 32 consecutive rows spread over the banks), the next step's global loads in flight
+// while the current one is multiplied. K % 8 == 0 and 16-byte aligned rows (host-checked).
+constexpr int MF_BK = 32, MF_LD = 40;
+template <int TM, int TN>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16* __restrict__ A, int lda, const bf16* __restrict__ W,
+                                                        int M, int N, int K, Epi e) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * MF_LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Ws[2][BN * MF_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int fr = lane & 31, fq = lane >> 5;
+  // staging: 4 threads per row (8 elements each), 64 rows per pass
+  const int sr = tid >> 2, sk = (tid & 3) * 8;
+  u32x4 ra[TM], rw[TN];
+  auto fetch = [&](int k0) {
+    const int k = k0 + sk;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m0 + sr + 64 * i;
+      ra[i] = (m < M && k < K) ? *(const u32x4*)(A + (long long)m * lda + k) : u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + sr + 64 * j;
+      rw[j] = (n < N && k < K) ? *(const u32x4*)(W + (long long)n * K + k) : u32x4{0, 0, 0, 0};
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) *(u32x4*)(&As[buf][(sr + 64 * i) * MF_LD + sk]) = ra[i];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) *(u32x4*)(&Ws[buf][(sr + 64 * j) * MF_LD + sk]) = rw[j];
+  };
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += MF_BK) {
+    const bool more = k0 + MF_BK < K;
+    if (more) fetch(k0 + MF_BK);
+#pragma unroll
+    for (int kk = 0; kk < MF_BK / 16; ++kk) {
+      bf16x8 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[i] = *(const bf16x8*)(&As[buf][(wm * 32 * TM + 32 * i + fr) * MF_LD + kk * 16 + fq * 8]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *(const bf16x8*)(&Ws[buf][(wn * 32 * TN + 32 * j + fr) * MF_LD + kk * 16 + fq * 8]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) stage(buf ^ 1);  // the other buffer's readers finished before the previous barrier
+    __syncthreads();
+    buf ^= 1;
+  }
+  // C fragment: column (weight row) = lane & 31, row (activation row) = (r & 3) + 8 (r >> 2) + 4 (lane >> 5)
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * 32 * TN + 32 * j + fr;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 * TM + 32 * i + (r & 3) + 8 * (r >> 2) + 4 * fq;
+        if (m < M && n < N) epi_store(e, m, n, acc[i][j][r]);
+      }
+    }
+}
+
+static int g_mfma = 1;
+void set_gemm_mfma(int on) { g_mfma = on; }
+
+int gemm_path(int M, int N, int K, int f32) {
+  if (M <= 8) return 0;
+  if (!f32 && g_mfma && K % 8 == 0) return 1;
+  return 2;
+}
+
+void gemm(const GemmParams& P, hipStream_t s) {
+  check(P.M > 0 && P.N > 0 && P.K > 0 && P.lda >= P.K && P.ldc >= P.N && P.A && P.W && P.C, "gemm: bad operands");
+  Epi e{P.epi, P.C, P.ldc, P.mult, P.add, P.cap};
+  int path = gemm_path(P.M, P.N, P.K, P.f32);
+  if (path == 1 && !(vec_ok<bf16>(P.A, P.lda, P.K) && vec_ok<bf16>(P.W, P.K, P.K))) path = 2;
+  if (path == 0) {
+    dim3 grid((P.N + 3) / 4);
+    if (P.f32) {
+      const int v = vec_ok<float>(P.A, P.lda, P.K) && vec_ok<float>(P.W, P.K, P.K);
+      hipLaunchKernelGGL(gemv_rows_kernel<float>, grid, dim3(256), 0, s, (const float*)P.A, P.lda, (const float*)P.W, P.M,
+                         P.N, P.K, e, v);
+    } else {
+      const int v = vec_ok<bf16>(P.A, P.lda, P.K) && vec_ok<bf16>(P.W, P.K, P.K);
+      hipLaunchKernelGGL(gemv_rows_kernel<bf16>, grid, dim3(256), 0, s, (const bf16*)P.A, P.lda, (const bf16*)P.W, P.M,
+                         P.N, P.K, e, v);
+    }
+  } else if (path == 1) {
+    // 128 x 128 tiles once they still fill the chip, else 64 x 64
+    const long long big = (long long)((P.M + 127) / 128) * ((P.N + 127) / 128);
+    if (big >= 256) {
+      dim3 grid((P.N + 127) / 128, (P.M + 127) / 128);
+      hipLaunchKernelGGL((gemm_mfma_kernel<2, 2>), grid, dim3(256), 0, s, (const bf16*)P.A, P.lda, (const bf16*)P.W, P.M,
+                         P.N, P.K, e);
+    } else {
+      dim3 grid((P.N + 63) / 64, (P.M + 63) / 64);
+      hipLaunchKernelGGL((gemm_mfma_kernel<1, 1>), grid, dim3(256), 0, s, (const bf16*)P.A, P.lda, (const bf16*)P.W, P.M,
+                         P.N, P.K, e);
+    }
+  } else {
+    dim3 grid((P.N + 63) / 64, (P.M + 63) / 64);
+    if (P.f32)
+      hipLaunchKernelGGL(gemm_fma_kernel<float>, grid, dim3(256), 0, s, (const float*)P.A, P.lda, (const float*)P.W, P.M,
+                         P.N, P.K, e);
+    else
+      hipLaunchKernelGGL(gemm_fma_kernel<bf16>, grid, dim3(256), 0, s, (const bf16*)P.A, P.lda, (const bf16*)P.W, P.M, P.N,
+                         P.K, e);
+  }
+  launched("gemm");
+}
+
+// ------------------------------------------------------------------------------------------------ embed / norm
+template <typename T>
+__global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, int E,
+                                                    int V, float* __restrict__ resid, float* __restrict__ x0) {
+  const int b = blockIdx.x;
+  int t = tokens[b];
+  t = t < 0 ? 0 : (t >= V ? V - 1 : t);
+  for (int i = threadIdx.x; i < E; i += 256) {
+    const float v = ld(table + (long long)t * E + i);
+    resid[(long long)b * E + i] = v;
+    x0[(long long)b * E + i] = v;
+  }
+}
+void embed(const void* table, const int* tokens, int B, int E, int V, float* resid, float* x0, int f32, hipStream_t s) {
+  check(B > 0 && table && tokens && resid && x0, "embed: bad operands");
+  if (f32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(B), dim3(256), 0, s, (const float*)table, tokens, E, V, resid, x0);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16>, dim3(B), dim3(256), 0, s, (const bf16*)table, tokens, E, V, resid, x0);
+  launched("embed");
+}
+
+// (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b, one block per row
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict__ x, const int* __restrict__ idx, int E,
+                                                         const float* __restrict__ w, const float* __restrict__ b,
+                                                         float eps, T* __restrict__ out) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const float* row = x + (long long)(idx ? idx[r] : r) * E;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < E; i += 256) sum += row[i];
+  const float mean = block_sum256(sum, red) / (float)E;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < E; i += 256) {
+    const float d = row[i] - mean;
+    sq += d * d;
+  }
+  const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)E + eps);
+  for (int i = threadIdx.x; i < E; i += 256) st(out + (long long)r * E + i, (row[i] - mean) * rstd * w[i] + b[i]);
+}
+void layer_norm_cast(const float* x, const int* idx, int rows, int E, const float* w, const float* b, float eps, void* out,
+                     int f32, hipStream_t s) {
+  check(rows > 0 && x && w && b && out, "layer_norm: bad operands");
+  if (f32)
+    hipLaunchKernelGGL(layer_norm_kernel<float>, dim3(rows), dim3(256), 0, s, x, idx, E, w, b, eps, (float*)out);
+  else
+    hipLaunchKernelGGL(layer_norm_kernel<bf16>, dim3(rows), dim3(256), 0, s, x, idx, E, w, b, eps, (bf16*)out);
+  launched("layer_norm");
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void concat_kernel(const float* __restrict__ x, const float* __restrict__ x0, int E,
+                                                     T* __restrict__ out) {
+  const int r = blockIdx.x;
+  for (int i = threadIdx.x; i < E; i += 256) {
+    st(out + (long long)r * 2 * E + i, x[(long long)r * E + i]);
+    st(out + (long long)r * 2 * E + E + i, x0[(long long)r * E + i]);
+  }
+}
+void concat_cast(const float* x, const float* x0, int rows, int E, void* out, int f32, hipStream_t s) {
+  check(rows > 0 && x && x0 && out, "concat: bad operands");
+  if (f32)
+    hipLaunchKernelGGL(concat_kernel<float>, dim3(rows), dim3(256), 0, s, x, x0, E, (float*)out);
+  else
+    hipLaunchKernelGGL(concat_kernel<bf16>, dim3(rows), dim3(256), 0, s, x, x0, E, (bf16*)out);
+  launched("concat");
+}
+
+// ------------------------------------------------------------------------------------------------ attention
+template <typename T>
+__global__ __launch_bounds__(256) void attn_prepare_kernel(AttnParams P, StepRows R) {
+  const int b = blockIdx.x;
+  float* row = P.proj + (long long)b * P.ld;
+  if (P.qtemp_coef != 0.f) {
+    const float p1 = (float)(R.pos[b] + 1);
+    const float temp = 1.f + P.qtemp_coef * logf(floorf(p1 / (float)P.qtemp_every) + 1.f);
+    for (int i = threadIdx.x; i < P.H * P.D; i += 256) row[P.off_q + i] *= temp;
+  }
+  const int slot = R.slot[b];
+  const long long blk = slot / R.bs, off = slot % R.bs;
+  T* kc = (T*)P.kc;
+  T* vc = (T*)P.vc;
+  for (int i = threadIdx.x; i < P.G * P.D; i += 256) {
+    const int g = i / P.D, d = i % P.D;
+    st(kc + ((blk * P.G + g) * R.bs + off) * P.D + d, row[P.off_k + i]);
+  }
+  for (int i = threadIdx.x; i < P.G * P.Dv; i += 256) {
+    const int g = i / P.Dv, d = i % P.Dv;
+    st(vc + ((blk * P.G + g) * R.bs + off) * P.Dv + d, row[P.off_v + i]);
+  }
+}
+void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s) {
+  check(R.B > 0 && P.proj && P.kc && P.vc, "attn_prepare: bad operands");
+  if (P.f32)
+    hipLaunchKernelGGL(attn_prepare_kernel<float>, dim3(R.B), dim3(256), 0, s, P, R);
+  else
+    hipLaunchKernelGGL(attn_prepare_kernel<bf16>, dim3(R.B), dim3(256), 0, s, P, R);
+  launched("attn_prepare");
+}
+
+// One wave per (row, head). Keys go by in groups of 64: lane j scores key t0 + j (its own K row), the wave
+// keeps a running maximum and sum, and every lane owns value dims lane, lane + 64, ... of the output.
+constexpr int ATT_MAXD = 256;
+template <typename T>
+__global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R) {
+  __shared__ float qs[4][ATT_MAXD];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int item = blockIdx.x * 4 + wv;
+  const bool live = item < R.B * P.H;
+  const int b = live ? item / P.H : 0, h = live ? item % P.H : 0;
+  const int g = h / (P.H / P.G);
+  const float* q = P.proj + (long long)b * P.ld + P.off_q + h * P.D;
+  for (int d = lane; d < P.D; d += 64) qs[wv][d] = live ? q[d] : 0.f;
+  __syncthreads();
+  if (!live) return;
+  const int n = R.q_len[b];
+  const int* bt = R.block_table + (long long)R.q_seq[b] * R.max_blocks;
+  const T* kc = (const T*)P.kc;
+  const T* vc = (const T*)P.vc;
+  float m = -INFINITY, l = 0.f;
+  float acc[ATT_MAXD / 64] = {};
+  for (int t0 = 0; t0 < n; t0 += 64) {
+    const int t = t0 + lane;
+    const bool valid = t < n;
+    int rowidx = 0;
+    float sc = -INFINITY;
+    if (valid) {
+      rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
+      const T* kr = kc + (long long)rowidx * P.D;
+      float dot = 0.f;
+      for (int d = 0; d < P.D; ++d) dot += qs[wv][d] * ld(kr + d);
+      sc = dot * P.scale;
+      if (P.softcap != 0.f) sc = P.softcap * tanhf(sc / P.softcap);
+    }
+    const float mn = fmaxf(m, wave_max(sc));
+    const float corr = expf(m - mn);  // first group: exp(-inf) = 0
+    const float p = valid ? expf(sc - mn) : 0.f;
+    l = l * corr + wave_sum(p);
+#pragma unroll
+    for (int c = 0; c < ATT_MAXD / 64; ++c) acc[c] *= corr;
+    m = mn;
+    const int cnt = min(64, n - t0);
+    for (int j = 0; j < cnt; ++j) {
+      const float pj = __shfl(p, j, 64);
+      const int rj = __shfl(rowidx, j, 64);
+      const T* vr = vc + (long long)rj * P.Dv;
+#pragma unroll
+      for (int c = 0; c < ATT_MAXD / 64; ++c) {
+        const int d = lane + 64 * c;
+        if (d < P.Dv) acc[c] += pj * ld(vr + d);
+      }
+    }
+  }
+  T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int c = 0; c < ATT_MAXD / 64; ++c) {
+    const int d = lane + 64 * c;
+    if (d < P.Dv) st(out + d, acc[c] * inv);
+  }
+}
+void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
+  check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && P.out,
+        "attention: head sizes up to 256, heads a multiple of key/value heads");
+  dim3 grid((R.B * P.H + 3) / 4);
+  if (P.f32)
+    hipLaunchKernelGGL(attention_kernel<float>, grid, dim3(256), 0, s, P, R);
+  else
+    hipLaunchKernelGGL(attention_kernel<bf16>, grid, dim3(256), 0, s, P, R);
+  launched("attention");
+}
+
+// ------------------------------------------------------------------------------------------------ retention
+// One block per (sequence segment of the step, head): the block of the segment's first row walks its rows in
+// order. Thread (g, j) = (tid / Dv, tid % Dv) holds state elements S[i][j] for i = g, g + NG, ... in registers
+// (NG = 256 / Dv thread groups), so the update S <- decay S + k v^T needs no communication and o = S^T q is a
+// sum of NG partials per column. Rotation of q and k, k's 1/sqrt(D), the per-head unit RMS of o and the
+// silu(g) gate are applied here; the state is read from and written back to its slot once per step.
+template <typename T, int MAXI>
+__global__ __launch_bounds__(256) void retention_kernel(RetParams P, StepRows R) {
+  __shared__ float qs[256], ks[256], vs[256], po[256], red[4];
+  const int r0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int seq = R.q_seq[r0];
+  if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;  // not the first row of its segment (uniform per block)
+  const int D = P.D, Dv = P.Dv;
+  const int NG = 256 / Dv;
+  const int g = tid / Dv, j = tid % Dv;
+  const bool act = g < NG;
+  float S[MAXI];
+  float* st_base = P.state + (((long long)seq * P.H + h) * D) * Dv;
+#pragma unroll
+  for (int ii = 0; ii < MAXI; ++ii) {
+    const int i = g + ii * NG;
+    S[ii] = (act && i < D) ? st_base[(long long)i * Dv + j] : 0.f;
+  }
+  const float dec = P.decay[h];
+  const float kscale = 1.f / sqrtf((float)D);
+  const int half = P.rot_dims / 2;
+  for (int r = r0; r < R.B && R.q_seq[r] == seq; ++r) {
+    const float* row = P.proj + (long long)r * P.ld;
+    if (tid < D) {
+      const float* q = row + P.off_q + h * D;
+      const float* k = row + P.off_k + h * D;
+      float qv = q[tid], kv = k[tid];
+      if (tid < P.rot_dims) {
+        const int i = tid < half ? tid : tid - half;
+        const float ang = (float)R.pos[r] * P.inv_freq[i];
+        const float c = cosf(ang), sn = sinf(ang);
+        if (tid < half) {  // (u, v) -> (u cos - v sin, v cos + u sin), u = x[i], v = x[i + half]
+          qv = q[tid] * c - q[tid + half] * sn;
+          kv = k[tid] * c - k[tid + half] * sn;
+        } else {
+          qv = q[tid] * c + q[i] * sn;
+          kv = k[tid] * c + k[i] * sn;
+        }
+      }
+      qs[tid] = qv;
+      ks[tid] = kv * kscale;
+    }
+    if (tid < Dv) vs[tid] = row[P.off_v + h * Dv + tid];
+    __syncthreads();
+    float part = 0.f;
+    if (act) {
+      const float vj = vs[j];
+#pragma unroll
+      for (int ii = 0; ii < MAXI; ++ii) {
+        const int i = g + ii * NG;
+        if (i < D) {
+          S[ii] = dec * S[ii] + ks[i] * vj;
+          part += S[ii] * qs[i];
+        }
+      }
+    }
+    po[tid] = part;
+    __syncthreads();
+    float o = 0.f;
+    if (tid < Dv)
+      for (int gg = 0; gg < NG; ++gg) o += po[gg * Dv + tid];
+    const float ms = block_sum256(tid < Dv ? o * o : 0.f, red) / (float)Dv;
+    if (tid < Dv) {
+      const float gate = row[P.off_g + h * Dv + tid];
+      st((T*)P.out + (long long)r * P.ld_out + h * Dv + tid, o / sqrtf(ms + P.eps) * silu(gate));
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int ii = 0; ii < MAXI; ++ii) {
+    const int i = g + ii * NG;
+    if (act && i < D) st_base[(long long)i * Dv + j] = S[ii];
+  }
+}
+bool retention_supported(int D, int Dv) {
+  if (D <= 0 || Dv <= 0 || D > 256 || Dv > 256) return false;
+  const int ng = 256 / Dv;
+  return (D + ng - 1) / ng <= 64;
+}
+template <typename T>
+static void launch_retention(const RetParams& P, const StepRows& R, hipStream_t s) {
+  const int ng = 256 / P.Dv, ni = (P.D + ng - 1) / ng;
+  dim3 grid(R.B, P.H);
+  if (ni <= 8)
+    hipLaunchKernelGGL((retention_kernel<T, 8>), grid, dim3(256), 0, s, P, R);
+  else if (ni <= 16)
+    hipLaunchKernelGGL((retention_kernel<T, 16>), grid, dim3(256), 0, s, P, R);
+  else if (ni <= 32)
+    hipLaunchKernelGGL((retention_kernel<T, 32>), grid, dim3(256), 0, s, P, R);
+  else
+    hipLaunchKernelGGL((retention_kernel<T, 64>), grid, dim3(256), 0, s, P, R);
+}
+void retention(const RetParams& P, const StepRows& R, hipStream_t s) {
+  check(R.B > 0 && P.proj && P.state && P.decay && P.out && retention_supported(P.D, P.Dv),
+        "retention: head sizes up to 256 with dim * vdim <= 16384");
+  check(P.rot_dims % 2 == 0 && P.rot_dims <= P.D && (P.rot_dims == 0 || P.inv_freq), "retention: bad rotary dims");
+  if (P.f32)
+    launch_retention<float>(P, R, s);
+  else
+    launch_retention<bf16>(P, R, s);
+  launched("retention");
+}
+
+// ------------------------------------------------------------------------------------------------ routed FFN
+// per row: the `top` largest router logits (ties: the lower expert), softmax over them; the shared expert's
+// scalar gate and its activation silu(gate) * up from the input projection's columns
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(MoeParams P) {
+  const int b = blockIdx.x;
+  const float* row = P.proj + (long long)b * P.ld;
+  if (threadIdx.x == 0) {
+    int ids[MOE_MAX_TOP];
+    float val[MOE_MAX_TOP];
+    for (int jj = 0; jj < P.top; ++jj) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int e = 0; e < P.X; ++e) {
+        bool taken = false;
+        for (int q = 0; q < jj; ++q) taken |= ids[q] == e;
+        if (taken) continue;
+        const float z = row[P.off_router + e] + P.router_b[e];
+        if (best < 0 || z > bv) {
+          best = e;
+          bv = z;
+        }
+      }
+      ids[jj] = best;
+      val[jj] = bv;
+    }
+    float sum = 0.f;
+    for (int jj = 0; jj < P.top; ++jj) {
+      val[jj] = expf(val[jj] - val[0]);
+      sum += val[jj];
+    }
+    for (int jj = 0; jj < P.top; ++jj) {
+      P.eids[(long long)b * P.ld_top + jj] = ids[jj];
+      P.ew[(long long)b * P.ld_top + jj] = val[jj] / sum;
+    }
+    if (P.Fs > 0) P.sgate[b] = sigmoidf(row[P.off_sg]);
+  }
+  T* hm = (T*)P.hmid + (long long)b * P.ld_hmid + P.top * P.F;
+  for (int f = threadIdx.x; f < P.Fs; f += 256) st(hm + f, silu(row[P.off_sgate + f]) * row[P.off_sup + f]);
+}
+// one wave per (row, routed expert, ff unit): gate and up rows of that expert meet the row's activations
+template <typename T>
+__global__ __launch_bounds__(256) void moe_experts_kernel(MoeParams P, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int b = blockIdx.y / P.top, jj = blockIdx.y % P.top;
+  if (f >= P.F) return;
+  const int e = P.eids[(long long)b * P.ld_top + jj];
+  const T* x = (const T*)P.h + (long long)b * P.E;
+  const T* wg = (const T*)P.w_gu + ((long long)e * 2 * P.F + f) * P.E;
+  const T* wu = wg + (long long)P.F * P.E;
+  const float gate = wave_dot<T>(wg, x, P.E, lane, vec != 0);
+  const float up = wave_dot<T>(wu, x, P.E, lane, vec != 0);
+  if (lane == 0) st((T*)P.hmid + (long long)b * P.ld_hmid + jj * P.F + f, silu(gate) * up);
+}
+// one wave per (row, output unit): the routed experts' down rows in routing order, then the shared expert's
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(MoeParams P, int vec, int vec_s) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int b = blockIdx.y;
+  if (n >= P.E) return;
+  const T* hm = (const T*)P.hmid + (long long)b * P.ld_hmid;
+  float y = 0.f;
+  for (int jj = 0; jj < P.top; ++jj) {
+    const int e = P.eids[(long long)b * P.ld_top + jj];
+    const T* wd = (const T*)P.w_down + ((long long)e * P.E + n) * P.F;
+    y += P.ew[(long long)b * P.ld_top + jj] * wave_dot<T>(wd, hm + jj * P.F, P.F, lane, vec != 0);
+  }
+  if (P.Fs > 0)
+    y += P.sgate[b] * wave_dot<T>((const T*)P.sh_down + (long long)n * P.Fs, hm + P.top * P.F, P.Fs, lane, vec_s != 0);
+  if (lane == 0) P.y[(long long)b * P.E + n] = y;
+}
+static void check_moe(const MoeParams& P) {
+  check(P.B > 0 && P.X > 0 && P.top > 0 && P.top <= P.X && P.top <= MOE_MAX_TOP && P.F > 0 && P.proj && P.h && P.w_gu &&
+            P.w_down && P.eids && P.ew && P.hmid && P.y && P.router_b && P.ld_top >= P.top &&
+            P.ld_hmid >= P.top * P.F + P.Fs && (P.Fs == 0 || (P.sh_down && P.sgate)),
+        "routed feed-forward: bad operands (top <= 16)");
+}
+void moe_route(const MoeParams& P, hipStream_t s) {
+  check_moe(P);
+  if (P.f32)
+    hipLaunchKernelGGL(moe_route_kernel<float>, dim3(P.B), dim3(256), 0, s, P);
+  else
+    hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(P.B), dim3(256), 0, s, P);
+  launched("moe_route");
+}
+void moe_experts(const MoeParams& P, hipStream_t s) {
+  check_moe(P);
+  dim3 grid((P.F + 3) / 4, P.B * P.top);
+  if (P.f32)
+    hipLaunchKernelGGL(moe_experts_kernel<float>, grid, dim3(256), 0, s, P,
+                       (int)(vec_ok<float>(P.h, P.E, P.E) && vec_ok<float>(P.w_gu, P.E, P.E)));
+  else
+    hipLaunchKernelGGL(moe_experts_kernel<bf16>, grid, dim3(256), 0, s, P,
+                       (int)(vec_ok<bf16>(P.h, P.E, P.E) && vec_ok<bf16>(P.w_gu, P.E, P.E)));
+  launched("moe_experts");
+}
+template <typename T>
+static void launch_moe_down(const MoeParams& P, hipStream_t s) {
+  // hmid rows: expert j's slice starts at j * F, the shared slice at top * F
+  const int v = vec_ok<T>(P.hmid, P.ld_hmid, P.F) && vec_ok<T>(P.w_down, P.F, P.F) && P.F % (16 / (int)sizeof(T)) == 0;
+  const int vs = P.Fs > 0 && v && vec_ok<T>(P.sh_down, P.Fs, P.Fs) && (P.top * P.F) % (16 / (int)sizeof(T)) == 0;
+  dim3 grid((P.E + 3) / 4, P.B);
+  hipLaunchKernelGGL(moe_down_kernel<T>, grid, dim3(256), 0, s, P, v, vs);
+}
+void moe_down(const MoeParams& P, hipStream_t s) {
+  check_moe(P);
+  if (P.f32)
+    launch_moe_down<float>(P, s);
+  else
+    launch_moe_down<bf16>(P, s);
+  launched("moe_down");
+}
+
+}  // namespace stack
+}  // namespace omx

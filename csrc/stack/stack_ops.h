@@ -1,0 +1,112 @@
+// Host-visible interface of the kernels of layer-list models (stack_kernels.hip): heterogeneous layers
+// with a float32 residual stream, matrices and K/V pools in bfloat16 or float32 (`f32` flag of every call),
+// paged softmax attention with capped scores and a query temperature, retention with a per-sequence state
+// matrix, and a routed feed-forward with a gated shared expert. Plain C++ types only.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+namespace omx {
+namespace stack {
+
+enum { EPI_STORE = 0, EPI_RESID = 1, EPI_SOFTCAP = 2 };
+
+// C = epi(A . W^T): A [M][K] (row stride lda) and W [N][K] in the matrix dtype, float32 accumulation.
+//   EPI_STORE:   C[m][n] = acc                                    (C float32, row stride ldc)
+//   EPI_RESID:   C[m][n] += mult * (acc + (add ? add[m][n] : 0))  (C = the residual stream; add stride ldc)
+//   EPI_SOFTCAP: C[m][n] = cap ? cap * tanh(acc / cap) : acc
+struct GemmParams {
+  const void* A;
+  int lda;
+  const void* W;
+  int M, N, K;
+  float* C;
+  int ldc;
+  int epi;
+  float mult;        // EPI_RESID
+  const float* add;  // EPI_RESID (or null)
+  float cap;         // EPI_SOFTCAP
+  int f32;           // matrices are float32 (else bfloat16)
+};
+void gemm(const GemmParams& P, hipStream_t s);
+// which kernel gemm() takes for these sizes: 0 wave-per-row GEMV (M <= 8), 1 matrix-core tile (bfloat16),
+// 2 FMA tile (float32, or a K that the vector loads do not cover)
+int gemm_path(int M, int N, int K, int f32);
+void set_gemm_mfma(int on);  // 0: bfloat16 tiles also take the FMA kernel (A/B and tests)
+
+void embed(const void* table, const int* tokens, int B, int E, int V, float* resid, float* x0, int f32, hipStream_t s);
+// out[r] = layer_norm(x[idx ? idx[r] : r]) * w + b, written in the matrix dtype
+void layer_norm_cast(const float* x, const int* idx, int rows, int E, const float* w, const float* b, float eps,
+                     void* out, int f32, hipStream_t s);
+// out[r] = [x[r]; x0[r]] in the matrix dtype, row stride 2E
+void concat_cast(const float* x, const float* x0, int rows, int E, void* out, int f32, hipStream_t s);
+
+struct StepRows {       // per-row step inputs (device arrays of B ints)
+  int B;
+  const int* pos;
+  const int* slot;      // flat cache slot (block * bs + offset)
+  const int* q_len;     // visible keys (pos + 1)
+  const int* q_seq;     // block-table row = state slot
+  const int* block_table;
+  int max_blocks, bs;
+};
+
+struct AttnParams {
+  float* proj;          // [B][ld] float32: q at off_q (scaled in place), k at off_k, v at off_v
+  int ld, off_q, off_k, off_v;
+  int H, G, D, Dv;
+  float scale, softcap, qtemp_coef;
+  int qtemp_every;
+  void* kc;             // [blocks][G][bs][D]
+  void* vc;             // [blocks][G][bs][Dv]
+  void* out;            // [B][ld_out] matrix dtype, head-major
+  int ld_out;
+  int f32;
+};
+// q *= 1 + coef * ln(floor((pos + 1) / every) + 1); k, v of every row stored at its slot
+void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s);
+// softmax(cap(q . k * scale)) v over the first q_len keys of the row's sequence
+void attention(const AttnParams& P, const StepRows& R, hipStream_t s);
+
+struct RetParams {
+  const float* proj;    // [B][ld] float32: q, k, v, g
+  int ld, off_q, off_k, off_v, off_g;
+  int H, D, Dv;
+  int rot_dims;         // rotate-half pairs (i, i + rot_dims / 2) on q and k
+  const float* inv_freq;  // [rot_dims / 2]
+  const float* decay;   // [H]
+  float* state;         // [slots][H][D][Dv] float32
+  float eps;
+  void* out;            // [B][ld_out] matrix dtype: unit_rms(o) * silu(g)
+  int ld_out;
+  int f32;
+};
+// rows of one sequence are contiguous and in position order; each sequence's state advances through them
+void retention(const RetParams& P, const StepRows& R, hipStream_t s);
+bool retention_supported(int D, int Dv);
+
+struct MoeParams {
+  const float* proj;    // [B][ld]: router logits at off_router, shared: scalar gate, gate rows, up rows
+  int ld, off_router, off_sg, off_sgate, off_sup;
+  int B, E, X, top, F, Fs;
+  const float* router_b;
+  const void* h;        // [B][E] matrix dtype (the normed activations)
+  const void* w_gu;     // [X][2F][E]
+  const void* w_down;   // [X][E][F]
+  const void* sh_down;  // [E][Fs]
+  int* eids;            // [B][ld_top]
+  float* ew;
+  int ld_top;
+  float* sgate;         // [B]
+  void* hmid;           // [B][ld_hmid] matrix dtype: top x F expert activations, then Fs shared
+  int ld_hmid;
+  float* y;             // [B][E] float32 feed-forward output
+  int f32;
+};
+void moe_route(const MoeParams& P, hipStream_t s);   // top-k ids + softmax weights, shared gate and activation
+void moe_experts(const MoeParams& P, hipStream_t s); // gate/up + activation of the routed experts -> hmid
+void moe_down(const MoeParams& P, hipStream_t s);    // y = sum_j w_j down_j(hmid_j) + sgate * shared_down(hmid_s)
+constexpr int MOE_MAX_TOP = 16;
+
+}  // namespace stack
+}  // namespace omx

@@ -380,7 +380,7 @@ class StackConfig:
                   loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
                   loop_times=int(loop.get("times", 0)) if loop else 0, norm_eps=float(c["norm"]["eps"]),
                   residual_mult=float(c.get("residual_mult", 1.0)), logit_softcap=float(c.get("logit_softcap") or 0.0),
-                  name=str(c.get("name", "bizulix")))
+                  name=str(c.get("name", "")))
         if cfg.loop_times and not 0 <= cfg.loop_start < cfg.loop_stop <= len(layers):
             raise UnsupportedArchitecture("loop: need 0 <= start < stop <= number of layers")
         return cfg
