@@ -349,8 +349,103 @@ def bench_tp(a) -> None:
     }), flush=True)
 
 
+STACK_SIZES = {
+    # name: width, layers (a = attention, r = retention), query heads, key/value heads, head dim, expert ff,
+    # experts, experts per token, shared-expert ff, retention heads x dim x vdim
+    "s": dict(E=1024, pattern="aaar" * 2, H=16, G=4, D=64, F=512, X=8, top=2, Fs=1024, ret=(8, 64, 128)),
+    "m": dict(E=2048, pattern="aaar" * 2, H=16, G=4, D=128, F=1024, X=8, top=2, Fs=2048, ret=(16, 64, 128)),
+}
+
+
+def stack_config(z: dict, vocab: int = 32000):
+    """A Bizulix model with the sizes of a real model's layers (random weights)."""
+    from ollama_operator_amd.models.config import (MIX_ATTENTION, MIX_RETENTION, LayerSpec, MixerSpec, MoESpec,
+                                                    StackConfig)
+    layers = []
+    for c in z["pattern"]:
+        if c == "a":
+            m = MixerSpec(kind=MIX_ATTENTION, heads=z["H"], kv_heads=z["G"], dim=z["D"], vdim=z["D"],
+                          scale=z["D"] ** -0.5, softcap=50.0, qtemp_coef=0.1, qtemp_every=1024)
+        else:
+            h, d, dv = z["ret"]
+            m = MixerSpec(kind=MIX_RETENTION, heads=h, kv_heads=h, dim=d, vdim=dv,
+                          decay=tuple(1.0 - 2.0 ** (-5 - i % 8) for i in range(h)), rot_dims=d, rot_base=1e4)
+        layers.append(LayerSpec(mixer=m, mlp=MoESpec(experts=z["X"], top=z["top"], ff=z["F"], shared_ff=z["Fs"])))
+    return StackConfig(n_vocab=vocab, n_embd=z["E"], layers=layers, norm_eps=1e-6, residual_mult=1.0, logit_softcap=30.0)
+
+
+def bench_stack(a) -> None:
+    """--stack SIZES: prefill and batch-1 decode throughput of the Bizulix design at sizes that resemble a real
+    model's layers, beside the closest GGUF model of the framework (Mixtral architecture, Q8_0) at equal width,
+    depth, heads, expert sizes and vocabulary. One JSON line; the default workload is not touched."""
+    import torch
+    from ollama_operator_amd.engine.runner import Runner
+    from ollama_operator_amd.engine.sampling import SamplingOptions
+    from ollama_operator_amd.engine.stack_runner import StackRunner
+    from ollama_operator_amd.gguf.constants import FileType
+    from ollama_operator_amd.models.config import ModelConfig
+    from ollama_operator_amd.models.random_init import write_random_gguf, write_random_stack
+    P, K, W = a.ttft_long or 2048, a.steps, a.warmup
+    ctx = P + K + W + 64
+    out = {}
+
+    def measure(r):
+        V = r.cfg.n_vocab
+        g = torch.Generator().manual_seed(5)
+        prompt = torch.randint(3, V, (P,), generator=g).tolist()
+        res = {}
+        for rep in range(2):  # the second pass is timed
+            sid = r.new_sequence()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            r.prefill(sid, prompt)
+            torch.cuda.synchronize()
+            res["prefill_tok_s"] = round(P / (time.perf_counter() - t0), 1)
+            if rep == 0:
+                r.free_sequence(sid)
+        gen = r.generate(r.new_sequence(), prompt[:a.prompt], SamplingOptions(seed=1), max_tokens=W + K + 8)
+        for _ in range(W + 1):
+            next(gen)
+        torch.cuda.synchronize()
+        s0, t0 = r.steps_issued, time.perf_counter()
+        while r.steps_issued - s0 < K:
+            next(gen)
+        torch.cuda.synchronize()
+        res["decode_tok_s"] = round((r.steps_issued - s0) / (time.perf_counter() - t0), 1)
+        res["ms_per_token"] = round(1e3 / res["decode_tok_s"], 4)
+        return res
+
+    for name in [x for x in a.stack.split(",") if x]:
+        z = STACK_SIZES[name]
+        d = os.path.join(a.dir, f"bizulix-{name}")
+        if not os.path.exists(os.path.join(d, "model.safetensors")):
+            write_random_stack(d, stack_config(z), seed=0, std=0.02)
+        r = StackRunner(d, device="cuda:0", dtype="bfloat16", max_batch=a.chunk, max_seqs=2, ctx=ctx)
+        r.warmup()
+        out[name] = {"bizulix_bf16": measure(r), "weights_gb": round(r.w.nbytes / 1e9, 3)}
+        r.close()
+        if not a.stack_only:
+            cfg = ModelConfig(name=f"mixtral-like-{name}", n_vocab=32000, n_embd=z["E"], n_layer=len(z["pattern"]),
+                              n_head=z["H"], n_head_kv=z["G"], n_ff=z["F"], n_rot=z["D"], n_embd_head=z["D"],
+                              ctx_len=max(4096, ctx), n_expert=z["X"], n_expert_used=z["top"])
+            path = os.path.join(a.dir, f"mixtral-like-{name}-q8_0.gguf")
+            if not os.path.exists(path):
+                write_random_gguf(path, cfg, FileType.MOSTLY_Q8_0, seed=0)
+            r = Runner(path, device="cuda:0", max_batch=a.chunk, max_seqs=2, ctx=ctx)
+            r.warmup()
+            out[name]["mixtral_like_q8_0"] = measure(r)
+            out[name]["mixtral_like_weights_gb"] = round(r.w.nbytes / 1e9, 3)
+            r.close()
+    print(json.dumps({"metric": "stack_throughput", "unit": "tokens/s", "prompt": P, "steps": K, "warmup": W,
+                      "dtype": "bf16", "data": "synthetic", "sizes": out}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--stack", default="", help="comma list of sizes (" + ", ".join(STACK_SIZES) + "): measure the "
+                    "Bizulix design at these sizes beside the closest GGUF model at equal size, instead of the "
+                    "default workload")
+    ap.add_argument("--stack-only", action="store_true", help="with --stack: skip the comparison model")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--tp", type=int, default=1, help="tensor-parallel degree: one sequence sharded over T GPUs")
     ap.add_argument("--allow-shared", action="store_true",
@@ -383,6 +478,9 @@ def main():
                     help="OLLAMA_NUM_PARALLEL of the spawned server (concurrent clients measured)")
     a = ap.parse_args()
     os.makedirs(a.dir, exist_ok=True)
+    if a.stack:
+        bench_stack(a)
+        return
     if a.tp > 1:
         bench_tp(a)
         return

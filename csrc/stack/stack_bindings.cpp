@@ -138,6 +138,18 @@ PYBIND11_MODULE(_stack, m) {
         w.ld_top = geti(d, "ld_top");
         w.sgate = Pp<float>(ptr(d, "sgate"));
         w.lrows = Pp<void>(ptr(d, "lrows"));
+        w.obuf = Pp<float>(ptr(d, "obuf"));
+        w.moe.rank = Pp<int>(ptr(d, "moe_rank"));
+        w.moe.srow = Pp<int>(ptr(d, "moe_srow"));
+        w.moe.inv = Pp<int>(ptr(d, "moe_inv"));
+        w.moe.tiles = Pp<int>(ptr(d, "moe_tiles"));
+        w.moe.ntiles = Pp<int>(ptr(d, "moe_ntiles"));
+        w.moe.gu = Pp<float>(ptr(d, "moe_gu"));
+        w.moe.hs = Pp<void>(ptr(d, "moe_hs"));
+        w.moe.ds = Pp<float>(ptr(d, "moe_ds"));
+        w.moe.max_pairs = geti(d, "moe_max_pairs");
+        w.moe.max_tiles = geti(d, "moe_max_tiles");
+        w.ld_obuf = geti(d, "ld_obuf");
       })
       .def("set_inputs", [](StackExecutor& e, py::dict d) {
         StackInputs& in = e.in;

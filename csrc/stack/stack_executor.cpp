@@ -65,16 +65,28 @@ void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
   } else {
     RetParams P{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.off_g, L.heads, L.dim, L.vdim, L.rot_dims, L.inv_freq,
                 L.decay, r.state, cfg.eps, ws.a, ws.ld_a, f32};
-    retention(P, R, s);
+    // prompt portions in chunks; a few rows (decode steps) token by token in one launch
+    if (B > SMALL_B && ws.obuf && ws.ld_obuf >= L.heads * L.vdim && retention_chunk_supported(L.dim, L.vdim))
+      retention_chunked(P, R, ws.obuf, ws.ld_obuf, s);
+    else
+      retention(P, R, s);
   }
   const float* ff = nullptr;
   if (L.experts) {
     MoeParams M{ws.proj, ws.ld_proj, L.off_router, L.off_sg, L.off_sgate, L.off_sup, B, E, L.experts, L.top, L.ff,
                 L.shared_ff, L.router_b, ws.h, L.w_gu, L.w_down, L.sh_down, ws.eids, ws.ew, ws.ld_top, ws.sgate, ws.hmid,
                 ws.ld_hmid, ws.y, f32};
+    if (B <= SMALL_B) {  // decode steps: two launches end the layer (residual update included)
+      moe_fused_small(M, ws.a, ws.ld_a, L.w_o, L.heads * L.vdim, ws.resid, cfg.residual_mult, s);
+      return;
+    }
     moe_route(M, s);
-    moe_experts(M, s);
-    moe_down(M, s);
+    if (ws.moe.gu && moe_grouped_supported(M)) {
+      moe_grouped(M, ws.moe, s);  // rows sorted by expert, one matrix-core product per expert tile
+    } else {
+      moe_experts(M, s);          // every pair streams its expert's rows once
+      moe_down(M, s);
+    }
     ff = ws.y;
   }
   // x <- x + m * (mixer output projection + feed-forward)

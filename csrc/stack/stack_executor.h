@@ -63,6 +63,9 @@ struct StackWorkspace {
   int ld_top = 0;
   float* sgate = nullptr;
   void* lrows = nullptr;   // [max_B][E] matrix dtype: normed rows for the head
+  MoeGroupWs moe{};        // grouped routed feed-forward (prompt portions, bfloat16); gu == null: unused
+  float* obuf = nullptr;   // [max_B][ld_obuf] float32: retention outputs before their norm (chunked path)
+  int ld_obuf = 0;
 };
 
 struct StackInputs {
@@ -77,6 +80,8 @@ struct StackInputs {
   int ld_logits = 0;
   const int* logit_idx = nullptr;
 };
+
+constexpr int SMALL_B = 16;  // steps of at most this many rows take the decode kernels
 
 class StackExecutor {
  public:

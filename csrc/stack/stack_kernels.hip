@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
 #include <stdexcept>
 #include <string>
 
@@ -189,25 +190,49 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const T* __restrict__ A, 
 // fragment reads of 32 consecutive rows spread over the banks), the next step's global loads in flight
 // while the current one is multiplied. K % 8 == 0 and 16-byte aligned rows (host-checked).
 constexpr int MF_BK = 32, MF_LD = 40;
+// Grouped form (routed experts): blockIdx.y walks a device-side table of row tiles {expert, first row, rows} over
+// rows sorted by expert; the tile's weight matrix is W + expert * w_stride, row m of the tile reads activation
+// row gather[m] / gdiv (or m itself) and writes output row m.
+struct Group {
+  const int* tiles;   // null: a plain product
+  const int* ntiles;
+  const int* gather;
+  int gdiv;
+  long long w_stride;
+};
 template <int TM, int TN>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16* __restrict__ A, int lda, const bf16* __restrict__ W,
-                                                        int M, int N, int K, Epi e) {
+                                                        int M, int N, int K, Epi e, Group G) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * MF_LD];
   __shared__ __attribute__((aligned(16))) uint16_t Ws[2][BN * MF_LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  int m0 = blockIdx.y * BM;
+  const int n0 = blockIdx.x * BN;
+  if (G.tiles) {
+    if ((int)blockIdx.y >= *G.ntiles) return;
+    const int* t = G.tiles + 3 * blockIdx.y;
+    W += (long long)t[0] * G.w_stride;
+    m0 = t[1];
+    M = t[1] + t[2];
+  }
   const int fr = lane & 31, fq = lane >> 5;
   // staging: 4 threads per row (8 elements each), 64 rows per pass
   const int sr = tid >> 2, sk = (tid & 3) * 8;
+  long long arow[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + sr + 64 * i;
+    arow[i] = (G.gather && m < M) ? G.gather[m] / G.gdiv : m;
+  }
   u32x4 ra[TM], rw[TN];
   auto fetch = [&](int k0) {
     const int k = k0 + sk;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int m = m0 + sr + 64 * i;
-      ra[i] = (m < M && k < K) ? *(const u32x4*)(A + (long long)m * lda + k) : u32x4{0, 0, 0, 0};
+      ra[i] = (m < M && k < K) ? *(const u32x4*)(A + arow[i] * lda + k) : u32x4{0, 0, 0, 0};
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -298,11 +323,11 @@ void gemm(const GemmParams& P, hipStream_t s) {
     if (big >= 256) {
       dim3 grid((P.N + 127) / 128, (P.M + 127) / 128);
       hipLaunchKernelGGL((gemm_mfma_kernel<2, 2>), grid, dim3(256), 0, s, (const bf16*)P.A, P.lda, (const bf16*)P.W, P.M,
-                         P.N, P.K, e);
+                         P.N, P.K, e, Group{});
     } else {
       dim3 grid((P.N + 63) / 64, (P.M + 63) / 64);
       hipLaunchKernelGGL((gemm_mfma_kernel<1, 1>), grid, dim3(256), 0, s, (const bf16*)P.A, P.lda, (const bf16*)P.W, P.M,
-                         P.N, P.K, e);
+                         P.N, P.K, e, Group{});
     }
   } else {
     dim3 grid((P.N + 63) / 64, (P.M + 63) / 64);
@@ -417,75 +442,213 @@ void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s) {
   launched("attn_prepare");
 }
 
-// One wave per (row, head). Keys go by in groups of 64: lane j scores key t0 + j (its own K row), the wave
-// keeps a running maximum and sum, and every lane owns value dims lane, lane + 64, ... of the output.
+// One wave per (row, key/value head, batch of up to RQ query heads that share it). Keys go by in groups of 64:
+// lane j reads the K row of key t0 + j once (16-byte loads) and scores it against every query head of the
+// batch; each head keeps a running maximum and sum; every lane owns value dims lane, lane + 64, ... of every
+// head's output, and a V row is read once for all of them.
 constexpr int ATT_MAXD = 256;
 template <typename T>
-__global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R) {
-  __shared__ float qs[4][ATT_MAXD];
+__device__ __forceinline__ void load8(const T* p, float* out);
+template <>
+__device__ __forceinline__ void load8<bf16>(const bf16* p, float* out) {
+  const u32x4 a = *(const u32x4*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = __uint_as_float(a[i] << 16);
+    out[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u);
+  }
+}
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, float* out) {
+  const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[i] = a[i];
+    out[4 + i] = b[i];
+  }
+}
+// DC = ceil(Dv / 64) value dims per lane. SPLIT: the block's four waves share ONE item and take the 64-key groups
+// in turn (few rows: decode steps), merging their running maxima, sums and outputs through LDS at the end;
+// otherwise every wave has its own item (prompt portions).
+template <typename T, int RQ, int DC, bool SPLIT>
+__global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R, int nbatch, int vec) {
+  __shared__ __attribute__((aligned(16))) float qs[SPLIT ? 1 : 4][RQ][ATT_MAXD];
+  __shared__ float mg[SPLIT ? 4 : 1][RQ][2];
+  __shared__ float ag[SPLIT ? 4 : 1][RQ][SPLIT ? DC * 64 : 1];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int item = blockIdx.x * 4 + wv;
-  const bool live = item < R.B * P.H;
-  const int b = live ? item / P.H : 0, h = live ? item % P.H : 0;
-  const int g = h / (P.H / P.G);
-  const float* q = P.proj + (long long)b * P.ld + P.off_q + h * P.D;
-  for (int d = lane; d < P.D; d += 64) qs[wv][d] = live ? q[d] : 0.f;
+  const int qw = SPLIT ? 0 : wv;
+  const int item = SPLIT ? blockIdx.x : blockIdx.x * 4 + wv;
+  const bool live = item < R.B * P.G * nbatch;
+  const int b = live ? item / (P.G * nbatch) : 0;
+  const int g = live ? (item / nbatch) % P.G : 0;
+  const int hb = live ? item % nbatch : 0;
+  const int per = P.H / P.G;
+  const int h0 = g * per + hb * RQ;            // first query head of this batch
+  const int nr = min(RQ, per - hb * RQ);       // heads in it
+  if (!SPLIT || wv == 0) {
+#pragma unroll
+    for (int r = 0; r < RQ; ++r)
+      for (int d = lane; d < P.D; d += 64)
+        qs[qw][r][d] = (live && r < nr) ? P.proj[(long long)b * P.ld + P.off_q + (h0 + r) * P.D + d] : 0.f;
+  }
   __syncthreads();
-  if (!live) return;
+  if (!live) return;  // SPLIT: uniform over the block
   const int n = R.q_len[b];
   const int* bt = R.block_table + (long long)R.q_seq[b] * R.max_blocks;
   const T* kc = (const T*)P.kc;
   const T* vc = (const T*)P.vc;
-  float m = -INFINITY, l = 0.f;
-  float acc[ATT_MAXD / 64] = {};
-  for (int t0 = 0; t0 < n; t0 += 64) {
+  float m[RQ], l[RQ], acc[RQ][DC];
+#pragma unroll
+  for (int r = 0; r < RQ; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) acc[r][c] = 0.f;
+  }
+  for (int t0 = SPLIT ? 64 * wv : 0; t0 < n; t0 += SPLIT ? 256 : 64) {
     const int t = t0 + lane;
     const bool valid = t < n;
     int rowidx = 0;
-    float sc = -INFINITY;
+    float dot[RQ];
+#pragma unroll
+    for (int r = 0; r < RQ; ++r) dot[r] = 0.f;
     if (valid) {
       rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
       const T* kr = kc + (long long)rowidx * P.D;
-      float dot = 0.f;
-      for (int d = 0; d < P.D; ++d) dot += qs[wv][d] * ld(kr + d);
-      sc = dot * P.scale;
-      if (P.softcap != 0.f) sc = P.softcap * tanhf(sc / P.softcap);
+      if (vec) {
+        for (int d = 0; d < P.D; d += 8) {
+          float k8[8];
+          load8<T>(kr + d, k8);
+#pragma unroll
+          for (int r = 0; r < RQ; ++r) {
+            const f32x4 qa = *(const f32x4*)&qs[qw][r][d], qb = *(const f32x4*)&qs[qw][r][d + 4];
+            dot[r] += qa[0] * k8[0] + qa[1] * k8[1] + qa[2] * k8[2] + qa[3] * k8[3] + qb[0] * k8[4] + qb[1] * k8[5] +
+                      qb[2] * k8[6] + qb[3] * k8[7];
+          }
+        }
+      } else {
+        for (int d = 0; d < P.D; ++d) {
+          const float kv = ld(kr + d);
+#pragma unroll
+          for (int r = 0; r < RQ; ++r) dot[r] += qs[qw][r][d] * kv;
+        }
+      }
     }
-    const float mn = fmaxf(m, wave_max(sc));
-    const float corr = expf(m - mn);  // first group: exp(-inf) = 0
-    const float p = valid ? expf(sc - mn) : 0.f;
-    l = l * corr + wave_sum(p);
+    float p[RQ];
 #pragma unroll
-    for (int c = 0; c < ATT_MAXD / 64; ++c) acc[c] *= corr;
-    m = mn;
+    for (int r = 0; r < RQ; ++r) {
+      float sc = -INFINITY;
+      if (valid) {
+        sc = dot[r] * P.scale;
+        if (P.softcap != 0.f) sc = P.softcap * tanhf(sc / P.softcap);
+      }
+      const float mn = fmaxf(m[r], wave_max(sc));
+      const float corr = expf(m[r] - mn);  // first group: exp(-inf) = 0
+      p[r] = valid ? expf(sc - mn) : 0.f;
+      l[r] = l[r] * corr + wave_sum(p[r]);
+#pragma unroll
+      for (int c = 0; c < DC; ++c) acc[r][c] *= corr;
+      m[r] = mn;
+    }
+    // values: 8 keys' rows in flight at a time (a key past the group's end reads row 0 with weight 0)
     const int cnt = min(64, n - t0);
-    for (int j = 0; j < cnt; ++j) {
-      const float pj = __shfl(p, j, 64);
-      const int rj = __shfl(rowidx, j, 64);
-      const T* vr = vc + (long long)rj * P.Dv;
+    for (int j0 = 0; j0 < cnt; j0 += 8) {
+      float v[8][DC];
 #pragma unroll
-      for (int c = 0; c < ATT_MAXD / 64; ++c) {
+      for (int u = 0; u < 8; ++u) {
+        const int rj = __shfl(rowidx, j0 + u, 64);
+        const T* vr = vc + (long long)rj * P.Dv;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) v[u][c] = (lane + 64 * c < P.Dv) ? ld(vr + lane + 64 * c) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int r = 0; r < RQ; ++r) {
+          const float pj = __shfl(p[r], j0 + u, 64);  // 0 for keys past the end
+#pragma unroll
+          for (int c = 0; c < DC; ++c) acc[r][c] += pj * v[u][c];
+        }
+    }
+  }
+  if (SPLIT) {
+#pragma unroll
+    for (int r = 0; r < RQ; ++r) {
+      if (lane == 0) {
+        mg[wv][r][0] = m[r];
+        mg[wv][r][1] = l[r];
+      }
+#pragma unroll
+      for (int c = 0; c < DC; ++c) ag[wv][r][lane + 64 * c] = acc[r][c];
+    }
+    __syncthreads();
+    if (wv != 0) return;
+#pragma unroll
+    for (int r = 0; r < RQ; ++r) {
+      float M = -INFINITY;
+      for (int w = 0; w < 4; ++w) M = fmaxf(M, mg[w][r][0]);
+      float L = 0.f;
+#pragma unroll
+      for (int c = 0; c < DC; ++c) acc[r][c] = 0.f;
+      for (int w = 0; w < 4; ++w) {
+        const float f = expf(mg[w][r][0] - M);  // a wave without keys: exp(-inf) = 0
+        L += mg[w][r][1] * f;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) acc[r][c] += ag[w][r][lane + 64 * c] * f;
+      }
+      l[r] = L;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RQ; ++r) {
+    if (r < nr) {
+      T* out = (T*)P.out + (long long)b * P.ld_out + (h0 + r) * P.Dv;
+      const float inv = 1.f / l[r];
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
         const int d = lane + 64 * c;
-        if (d < P.Dv) acc[c] += pj * ld(vr + d);
+        if (d < P.Dv) st(out + d, acc[r][c] * inv);
       }
     }
   }
-  T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
-  const float inv = 1.f / l;
-#pragma unroll
-  for (int c = 0; c < ATT_MAXD / 64; ++c) {
-    const int d = lane + 64 * c;
-    if (d < P.Dv) st(out + d, acc[c] * inv);
-  }
+}
+template <typename T, int RQ, int DC>
+static void launch_attention_rd(const AttnParams& P, const StepRows& R, int nbatch, int vec, hipStream_t s) {
+  const int items = R.B * P.G * nbatch;
+  if (items < 512)
+    hipLaunchKernelGGL((attention_kernel<T, RQ, DC, true>), dim3(items), dim3(256), 0, s, P, R, nbatch, vec);
+  else
+    hipLaunchKernelGGL((attention_kernel<T, RQ, DC, false>), dim3((items + 3) / 4), dim3(256), 0, s, P, R, nbatch, vec);
+}
+template <typename T, int RQ>
+static void launch_attention_r(const AttnParams& P, const StepRows& R, int nbatch, int vec, hipStream_t s) {
+  if (P.Dv <= 64)
+    launch_attention_rd<T, RQ, 1>(P, R, nbatch, vec, s);
+  else if (P.Dv <= 128)
+    launch_attention_rd<T, RQ, 2>(P, R, nbatch, vec, s);
+  else
+    launch_attention_rd<T, RQ, 4>(P, R, nbatch, vec, s);
+}
+template <typename T>
+static void launch_attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
+  const int per = P.H / P.G;
+  const int rq = per >= 4 ? 4 : per >= 2 ? 2 : 1;
+  const int nbatch = (per + rq - 1) / rq;
+  const int vec = P.D % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
+  if (rq == 4)
+    launch_attention_r<T, 4>(P, R, nbatch, vec, s);
+  else if (rq == 2)
+    launch_attention_r<T, 2>(P, R, nbatch, vec, s);
+  else
+    launch_attention_r<T, 1>(P, R, nbatch, vec, s);
 }
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && P.out,
         "attention: head sizes up to 256, heads a multiple of key/value heads");
-  dim3 grid((R.B * P.H + 3) / 4);
   if (P.f32)
-    hipLaunchKernelGGL(attention_kernel<float>, grid, dim3(256), 0, s, P, R);
+    launch_attention<float>(P, R, s);
   else
-    hipLaunchKernelGGL(attention_kernel<bf16>, grid, dim3(256), 0, s, P, R);
+    launch_attention<bf16>(P, R, s);
   launched("attention");
 }
 
@@ -568,6 +731,167 @@ __global__ __launch_bounds__(256) void retention_kernel(RetParams P, StepRows R)
     if (act && i < D) st_base[(long long)i * Dv + j] = S[ii];
   }
 }
+// Prompt portions: the same recurrence in chunks of RC tokens. With g the head's decay, a chunk that starts
+// from state S computes, for its tokens t, s = 0 .. n - 1,
+//   A[t][s] = (q_t . k_s) g^(t - s) for s <= t,   o_t = g^(t + 1) S^T q_t + sum_s A[t][s] v_s,
+//   S <- g^n S + sum_s g^(n - 1 - s) k_s v_s^T,
+// all in float32 on the vector ALUs. One block per (segment, head, 64 value columns): thread (g4, j) keeps
+// column j of S in registers, produces o_t[j] for t = g4, g4 + 4, ..., and the four threads of a column advance
+// their copies of it alike. The un-normalised o goes to `obuf`; retention_finish_kernel applies the per-head
+// unit RMS and the gate.
+constexpr int RC = 32;
+template <int MAXD>
+__global__ __launch_bounds__(256) void retention_chunk_kernel(RetParams P, StepRows R, float* __restrict__ obuf,
+                                                              int ld_o, int NJ) {
+  __shared__ __attribute__((aligned(16))) float Qs[RC][MAXD];
+  __shared__ __attribute__((aligned(16))) float Ks[RC][MAXD + 4];
+  __shared__ float Vs[RC][64];
+  __shared__ float As[RC][RC + 1];
+  __shared__ float pw[RC + 1];
+  __shared__ int seg_n;
+  const int r0 = blockIdx.x, h = blockIdx.y / NJ, jb = blockIdx.y % NJ, tid = threadIdx.x;
+  const int seq = R.q_seq[r0];
+  if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;
+  const int D = P.D, Dv = P.Dv;
+  const int j = tid & 63, g4 = tid >> 6;
+  const int col = jb * 64 + j;
+  const bool colok = col < Dv;
+  const float dec = P.decay[h];
+  if (tid == 0) seg_n = R.B - r0;
+  if (tid <= RC) pw[tid] = powf(dec, (float)tid);
+  __syncthreads();
+  for (int i = 1 + tid; r0 + i < R.B; i += 256)  // the segment ends at the first row of another sequence
+    if (R.q_seq[r0 + i] != seq) {
+      atomicMin(&seg_n, i);
+      break;
+    }
+  float S[MAXD];
+  float* st_base = P.state + (((long long)seq * P.H + h) * D) * Dv;
+#pragma unroll
+  for (int i = 0; i < MAXD; ++i) S[i] = (colok && i < D) ? st_base[(long long)i * Dv + col] : 0.f;
+  __syncthreads();
+  const int n = seg_n;
+  const float kscale = 1.f / sqrtf((float)D);
+  const int half = P.rot_dims / 2;
+  for (int c0 = 0; c0 < n; c0 += RC) {
+    const int cn = min(RC, n - c0);
+    // stage the chunk: rows past cn and dims past D are zero, so the loops below run to their full extent
+    for (int idx = tid; idx < RC * MAXD; idx += 256) {
+      const int c = idx / MAXD, d = idx % MAXD;
+      float qv = 0.f, kv = 0.f;
+      if (c < cn && d < D) {
+        const int r = r0 + c0 + c;
+        const float* q = P.proj + (long long)r * P.ld + P.off_q + h * D;
+        const float* k = P.proj + (long long)r * P.ld + P.off_k + h * D;
+        qv = q[d];
+        kv = k[d];
+        if (d < P.rot_dims) {
+          const int i = d < half ? d : d - half;
+          const float ang = (float)R.pos[r] * P.inv_freq[i];
+          const float cs = cosf(ang), sn = sinf(ang);
+          if (d < half) {
+            qv = q[d] * cs - q[d + half] * sn;
+            kv = k[d] * cs - k[d + half] * sn;
+          } else {
+            qv = q[d] * cs + q[i] * sn;
+            kv = k[d] * cs + k[i] * sn;
+          }
+        }
+      }
+      Qs[c][d] = qv;
+      Ks[c][d] = kv * kscale;
+    }
+    for (int idx = tid; idx < RC * 64; idx += 256) {
+      const int c = idx >> 6, jj = idx & 63;
+      const int cc = jb * 64 + jj;
+      Vs[c][jj] = (c < cn && cc < Dv) ? P.proj[(long long)(r0 + c0 + c) * P.ld + P.off_v + h * Dv + cc] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kx = 0; kx < RC * RC / 256; ++kx) {
+      const int t = (tid >> 5) + 8 * kx, sx = tid & 31;
+      float dot = 0.f;
+      if (sx <= t) {
+#pragma unroll
+        for (int i4 = 0; i4 < MAXD / 4; ++i4) {
+          const f32x4 a = *(const f32x4*)&Qs[t][4 * i4], b = *(const f32x4*)&Ks[sx][4 * i4];
+          dot += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+        }
+        dot *= pw[t - sx];
+      }
+      As[t][sx] = dot;
+    }
+    __syncthreads();
+    for (int t = g4; t < cn; t += 4) {
+      float inter = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < MAXD / 4; ++i4) {
+        const f32x4 a = *(const f32x4*)&Qs[t][4 * i4];
+        inter += a[0] * S[4 * i4] + a[1] * S[4 * i4 + 1] + a[2] * S[4 * i4 + 2] + a[3] * S[4 * i4 + 3];
+      }
+      float intra = 0.f;
+#pragma unroll
+      for (int sx = 0; sx < RC; ++sx) intra += As[t][sx] * Vs[sx][j];  // As is zero above the diagonal
+      if (colok) obuf[(long long)(r0 + c0 + t) * ld_o + h * Dv + col] = pw[t + 1] * inter + intra;
+    }
+    const float dn = pw[cn];
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i) S[i] *= dn;
+    for (int sx = 0; sx < cn; ++sx) {
+      const float vv = Vs[sx][j] * pw[cn - 1 - sx];
+#pragma unroll
+      for (int i4 = 0; i4 < MAXD / 4; ++i4) {
+        const f32x4 b = *(const f32x4*)&Ks[sx][4 * i4];
+        S[4 * i4] += b[0] * vv;
+        S[4 * i4 + 1] += b[1] * vv;
+        S[4 * i4 + 2] += b[2] * vv;
+        S[4 * i4 + 3] += b[3] * vv;
+      }
+    }
+    __syncthreads();
+  }
+  if (g4 == 0 && colok) {
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i)
+      if (i < D) st_base[(long long)i * Dv + col] = S[i];
+  }
+}
+// out = o / sqrt(mean_j(o^2) + eps) * silu(gate), one wave per (row, head)
+template <typename T>
+__global__ __launch_bounds__(256) void retention_finish_kernel(RetParams P, int B, const float* __restrict__ obuf,
+                                                               int ld_o) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= B * P.H) return;
+  const int b = item / P.H, h = item % P.H;
+  const float* o = obuf + (long long)b * ld_o + h * P.Dv;
+  float sq = 0.f;
+  for (int jx = lane; jx < P.Dv; jx += 64) sq += o[jx] * o[jx];
+  const float rs = 1.f / sqrtf(wave_sum(sq) / (float)P.Dv + P.eps);
+  const float* gate = P.proj + (long long)b * P.ld + P.off_g + h * P.Dv;
+  T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
+  for (int jx = lane; jx < P.Dv; jx += 64) st(out + jx, o[jx] * rs * silu(gate[jx]));
+}
+bool retention_chunk_supported(int D, int Dv) { return D > 0 && D <= 128 && Dv > 0 && Dv <= 256; }
+void retention_chunked(const RetParams& P, const StepRows& R, float* obuf, int ld_o, hipStream_t s) {
+  check(R.B > 0 && P.proj && P.state && P.decay && P.out && obuf && ld_o >= P.H * P.Dv && retention_chunk_supported(P.D, P.Dv),
+        "chunked retention: dim <= 128, vdim <= 256");
+  check(P.rot_dims % 2 == 0 && P.rot_dims <= P.D && (P.rot_dims == 0 || P.inv_freq), "retention: bad rotary dims");
+  const int NJ = (P.Dv + 63) / 64;
+  dim3 grid(R.B, P.H * NJ);
+  if (P.D <= 64)
+    hipLaunchKernelGGL(retention_chunk_kernel<64>, grid, dim3(256), 0, s, P, R, obuf, ld_o, NJ);
+  else
+    hipLaunchKernelGGL(retention_chunk_kernel<128>, grid, dim3(256), 0, s, P, R, obuf, ld_o, NJ);
+  launched("retention_chunk");
+  dim3 g2((R.B * P.H + 3) / 4);
+  if (P.f32)
+    hipLaunchKernelGGL(retention_finish_kernel<float>, g2, dim3(256), 0, s, P, R.B, obuf, ld_o);
+  else
+    hipLaunchKernelGGL(retention_finish_kernel<bf16>, g2, dim3(256), 0, s, P, R.B, obuf, ld_o);
+  launched("retention_finish");
+}
+
 bool retention_supported(int D, int Dv) {
   if (D <= 0 || Dv <= 0 || D > 256 || Dv > 256) return false;
   const int ng = 256 / Dv;
@@ -623,9 +947,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(MoeParams P) {
       ids[jj] = best;
       val[jj] = bv;
     }
+    const float mx = val[0];  // picked first: the largest
     float sum = 0.f;
     for (int jj = 0; jj < P.top; ++jj) {
-      val[jj] = expf(val[jj] - val[0]);
+      val[jj] = expf(val[jj] - mx);
       sum += val[jj];
     }
     for (int jj = 0; jj < P.top; ++jj) {
@@ -670,6 +995,233 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeParams P, int vec, int
     y += P.sgate[b] * wave_dot<T>((const T*)P.sh_down + (long long)n * P.Fs, hm + P.top * P.F, P.Fs, lane, vec_s != 0);
   if (lane == 0) P.y[(long long)b * P.E + n] = y;
 }
+// ---- prompt portions: pairs (row, routed expert) sorted by expert, one matrix-core product per expert tile
+// One block: counts per expert (LDS atomics hand every pair its rank inside its expert; the order inside an
+// expert does not reach the result, every pair's output row is its own), offsets, the tile table, and the two
+// maps sorted position -> pair and pair -> sorted position.
+__global__ __launch_bounds__(256) void moe_sort_kernel(const int* __restrict__ eids, int ld_top, int B, int top, int X,
+                                                       int tile_m, int* __restrict__ rank, int* __restrict__ srow,
+                                                       int* __restrict__ inv, int* __restrict__ tiles,
+                                                       int* __restrict__ ntiles) {
+  __shared__ int cnt[256], off[256];
+  const int tid = threadIdx.x, P = B * top;
+  for (int e = tid; e < X; e += 256) cnt[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < P; p += 256) rank[p] = atomicAdd(&cnt[eids[(long long)(p / top) * ld_top + p % top]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < X; ++e) {
+      off[e] = at;
+      for (int t0 = 0; t0 < cnt[e]; t0 += tile_m) {
+        tiles[3 * nt] = e;
+        tiles[3 * nt + 1] = at + t0;
+        tiles[3 * nt + 2] = min(tile_m, cnt[e] - t0);
+        ++nt;
+      }
+      at += cnt[e];
+    }
+    *ntiles = nt;
+  }
+  __syncthreads();
+  for (int p = tid; p < P; p += 256) {
+    const int pos = off[eids[(long long)(p / top) * ld_top + p % top]] + rank[p];
+    srow[pos] = p;
+    inv[p] = pos;
+  }
+}
+// hs[pos][f] = silu(gu[pos][f]) * gu[pos][F + f], in the matrix dtype
+__global__ __launch_bounds__(256) void moe_act_kernel(const float* __restrict__ gu, int P, int F, bf16* __restrict__ hs) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)P * F) return;
+  const long long pos = i / F;
+  const int f = (int)(i % F);
+  st(hs + i, silu(gu[pos * 2 * F + f]) * gu[pos * 2 * F + F + f]);
+}
+// y[b][n] = (shared ? sgate[b] * y[b][n] : 0) + sum_j ew[b][j] * ds[inv[b * top + j]][n], routing order
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ ds,
+                                                          const int* __restrict__ inv, const float* __restrict__ ew,
+                                                          int ld_top, const float* __restrict__ sgate, int B, int E, int top,
+                                                          int shared) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)B * E) return;
+  const int b = (int)(i / E), n = (int)(i % E);
+  float acc = shared ? sgate[b] * y[i] : 0.f;
+  float routed = 0.f;
+  for (int j = 0; j < top; ++j) routed += ew[(long long)b * ld_top + j] * ds[(long long)inv[b * top + j] * E + n];
+  y[i] = routed + acc;
+}
+bool moe_grouped_supported(const MoeParams& P) {
+  return !P.f32 && P.X <= 256 && P.E % 8 == 0 && P.F % 8 == 0 && (P.Fs == 0 || (P.Fs % 8 == 0 && (P.top * P.F) % 8 == 0 &&
+         P.ld_hmid % 8 == 0));
+}
+void moe_grouped(const MoeParams& P, const MoeGroupWs& W, hipStream_t s) {
+  check(moe_grouped_supported(P) && W.rank && W.srow && W.inv && W.tiles && W.ntiles && W.gu && W.hs && W.ds,
+        "grouped routed feed-forward: workspace or sizes");
+  const int pairs = P.B * P.top;
+  const int tile_m = pairs / P.X >= 192 ? 128 : 64;
+  const int max_tiles = (pairs + tile_m - 1) / tile_m + P.X;
+  check(pairs <= W.max_pairs && max_tiles <= W.max_tiles, "grouped routed feed-forward: workspace too small");
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(256), 0, s, P.eids, P.ld_top, P.B, P.top, P.X, tile_m, W.rank, W.srow,
+                     W.inv, W.tiles, W.ntiles);
+  launched("moe_sort");
+  // gate | up of every pair with its expert's matrix
+  {
+    Epi e{EPI_STORE, W.gu, 2 * P.F, 0.f, nullptr, 0.f};
+    Group G{W.tiles, W.ntiles, W.srow, P.top, (long long)2 * P.F * P.E};
+    if (tile_m == 128) {
+      dim3 grid((2 * P.F + 127) / 128, max_tiles);
+      hipLaunchKernelGGL((gemm_mfma_kernel<2, 2>), grid, dim3(256), 0, s, (const bf16*)P.h, P.E, (const bf16*)P.w_gu, pairs,
+                         2 * P.F, P.E, e, G);
+    } else {
+      dim3 grid((2 * P.F + 63) / 64, max_tiles);
+      hipLaunchKernelGGL((gemm_mfma_kernel<1, 1>), grid, dim3(256), 0, s, (const bf16*)P.h, P.E, (const bf16*)P.w_gu, pairs,
+                         2 * P.F, P.E, e, G);
+    }
+    launched("moe_gemm gate/up");
+  }
+  {
+    const long long n = (long long)pairs * P.F;
+    hipLaunchKernelGGL(moe_act_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, W.gu, pairs, P.F, (bf16*)W.hs);
+    launched("moe_act");
+  }
+  {
+    Epi e{EPI_STORE, W.ds, P.E, 0.f, nullptr, 0.f};
+    Group G{W.tiles, W.ntiles, nullptr, 1, (long long)P.E * P.F};
+    if (tile_m == 128) {
+      dim3 grid((P.E + 127) / 128, max_tiles);
+      hipLaunchKernelGGL((gemm_mfma_kernel<2, 2>), grid, dim3(256), 0, s, (const bf16*)W.hs, P.F, (const bf16*)P.w_down, pairs,
+                         P.E, P.F, e, G);
+    } else {
+      dim3 grid((P.E + 63) / 64, max_tiles);
+      hipLaunchKernelGGL((gemm_mfma_kernel<1, 1>), grid, dim3(256), 0, s, (const bf16*)W.hs, P.F, (const bf16*)P.w_down, pairs,
+                         P.E, P.F, e, G);
+    }
+    launched("moe_gemm down");
+  }
+  if (P.Fs > 0) {  // the shared expert's down projection over every row, into y
+    GemmParams g{(const bf16*)P.hmid + P.top * P.F, P.ld_hmid, P.sh_down, P.B, P.E, P.Fs, P.y, P.E, EPI_STORE, 0.f, nullptr,
+                 0.f, 0};
+    gemm(g, s);
+  }
+  {
+    const long long n = (long long)P.B * P.E;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, P.y, W.ds, W.inv, P.ew, P.ld_top,
+                       P.sgate, P.B, P.E, P.top, (int)(P.Fs > 0));
+    launched("moe_combine");
+  }
+}
+
+// ---- a few rows (decode steps): two launches for the whole feed-forward and the layer's residual update
+// Routing of one row by one thread (the caller's thread 0): ids and weights into LDS arrays
+__device__ __forceinline__ void route_row(const MoeParams& P, const float* row, int* ids, float* val) {
+  for (int jj = 0; jj < P.top; ++jj) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < P.X; ++e) {
+      bool taken = false;
+      for (int q = 0; q < jj; ++q) taken |= ids[q] == e;
+      if (taken) continue;
+      const float z = row[P.off_router + e] + P.router_b[e];
+      if (best < 0 || z > bv) {
+        best = e;
+        bv = z;
+      }
+    }
+    ids[jj] = best;
+    val[jj] = bv;
+  }
+  const float mx = val[0];
+  float sum = 0.f;
+  for (int jj = 0; jj < P.top; ++jj) {
+    val[jj] = expf(val[jj] - mx);
+    sum += val[jj];
+  }
+  for (int jj = 0; jj < P.top; ++jj) val[jj] /= sum;
+}
+// grid (ceil(max(F, Fs) / 4), B * (top + 1)): blocks y = b * (top + 1) + jj route row b again (a few dozen
+// operations) and take routed expert jj < top, or (jj == top) the shared expert's activation from the input
+// projection; the first block of a row also leaves ids, weights and the shared gate for the second launch
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_experts_kernel(MoeParams P, int vec) {
+  __shared__ int ids[MOE_MAX_TOP];
+  __shared__ float val[MOE_MAX_TOP];
+  const int lane = threadIdx.x & 63;
+  const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int b = blockIdx.y / (P.top + 1), jj = blockIdx.y % (P.top + 1);
+  const float* row = P.proj + (long long)b * P.ld;
+  T* hm = (T*)P.hmid + (long long)b * P.ld_hmid;
+  if (jj == P.top) {  // shared expert
+    if (f < P.Fs && lane == 0) st(hm + P.top * P.F + f, silu(row[P.off_sgate + f]) * row[P.off_sup + f]);
+    return;
+  }
+  if (threadIdx.x == 0) {
+    route_row(P, row, ids, val);
+    if (blockIdx.x == 0 && jj == 0) {
+      for (int q = 0; q < P.top; ++q) {
+        P.eids[(long long)b * P.ld_top + q] = ids[q];
+        P.ew[(long long)b * P.ld_top + q] = val[q];
+      }
+      if (P.Fs > 0) P.sgate[b] = sigmoidf(row[P.off_sg]);
+    }
+  }
+  __syncthreads();
+  if (f >= P.F) return;
+  const int e = ids[jj];
+  const T* x = (const T*)P.h + (long long)b * P.E;
+  const T* wg = (const T*)P.w_gu + ((long long)e * 2 * P.F + f) * P.E;
+  const T* wu = wg + (long long)P.F * P.E;
+  const float gate = wave_dot<T>(wg, x, P.E, lane, vec != 0);
+  const float up = wave_dot<T>(wu, x, P.E, lane, vec != 0);
+  if (lane == 0) st(hm + jj * P.F + f, silu(gate) * up);
+}
+// x[b][n] += mult * (W_o[n] . a[b] + sum_j w_j W_down[e_j][n] . hmid_j + sgate * W_shared_down[n] . hmid_s):
+// one wave per output unit, every row of the step
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_out_kernel(MoeParams P, const T* __restrict__ a, int lda,
+                                                           const T* __restrict__ w_o, int Ko, float* __restrict__ x,
+                                                           float mult, int vec, int vec_s, int vec_o) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= P.E) return;
+  for (int b = 0; b < P.B; ++b) {
+    float y = wave_dot<T>(w_o + (long long)n * Ko, a + (long long)b * lda, Ko, lane, vec_o != 0);
+    const T* hm = (const T*)P.hmid + (long long)b * P.ld_hmid;
+    for (int jj = 0; jj < P.top; ++jj) {
+      const int e = P.eids[(long long)b * P.ld_top + jj];
+      const T* wd = (const T*)P.w_down + ((long long)e * P.E + n) * P.F;
+      y += P.ew[(long long)b * P.ld_top + jj] * wave_dot<T>(wd, hm + jj * P.F, P.F, lane, vec != 0);
+    }
+    if (P.Fs > 0)
+      y += P.sgate[b] * wave_dot<T>((const T*)P.sh_down + (long long)n * P.Fs, hm + P.top * P.F, P.Fs, lane, vec_s != 0);
+    if (lane == 0) x[(long long)b * P.E + n] += mult * y;
+  }
+}
+static void check_moe(const MoeParams& P);
+template <typename T>
+static void launch_moe_fused(const MoeParams& P, const void* a, int lda, const void* w_o, int Ko, float* x, float mult,
+                             hipStream_t s) {
+  const int per = 16 / (int)sizeof(T);
+  const int v1 = vec_ok<T>(P.h, P.E, P.E) && vec_ok<T>(P.w_gu, P.E, P.E);
+  dim3 g1((std::max(P.F, P.Fs) + 3) / 4, P.B * (P.top + 1));
+  hipLaunchKernelGGL(moe_route_experts_kernel<T>, g1, dim3(256), 0, s, P, v1);
+  const int v = vec_ok<T>(P.hmid, P.ld_hmid, P.F) && vec_ok<T>(P.w_down, P.F, P.F);
+  const int vs = P.Fs > 0 && vec_ok<T>(P.hmid, P.ld_hmid, P.Fs) && vec_ok<T>(P.sh_down, P.Fs, P.Fs) && (P.top * P.F) % per == 0;
+  const int vo = vec_ok<T>(a, lda, Ko) && vec_ok<T>(w_o, Ko, Ko);
+  dim3 g2((P.E + 3) / 4);
+  hipLaunchKernelGGL(moe_down_out_kernel<T>, g2, dim3(256), 0, s, P, (const T*)a, lda, (const T*)w_o, Ko, x, mult, v, vs, vo);
+}
+void moe_fused_small(const MoeParams& P, const void* a, int lda, const void* w_o, int Ko, float* x, float mult,
+                     hipStream_t s) {
+  check_moe(P);
+  check(a && w_o && x && Ko > 0 && lda >= Ko, "fused feed-forward + output projection: bad operands");
+  if (P.f32)
+    launch_moe_fused<float>(P, a, lda, w_o, Ko, x, mult, s);
+  else
+    launch_moe_fused<bf16>(P, a, lda, w_o, Ko, x, mult, s);
+  launched("moe_fused_small");
+}
+
 static void check_moe(const MoeParams& P) {
   check(P.B > 0 && P.X > 0 && P.top > 0 && P.top <= P.X && P.top <= MOE_MAX_TOP && P.F > 0 && P.proj && P.h && P.w_gu &&
             P.w_down && P.eids && P.ew && P.hmid && P.y && P.router_b && P.ld_top >= P.top &&

@@ -84,6 +84,10 @@ struct RetParams {
 // rows of one sequence are contiguous and in position order; each sequence's state advances through them
 void retention(const RetParams& P, const StepRows& R, hipStream_t s);
 bool retention_supported(int D, int Dv);
+// the same recurrence in chunks (prompt portions): un-normalised o into obuf [B][ld_o] float32, then the unit
+// RMS and the gate in a second launch
+void retention_chunked(const RetParams& P, const StepRows& R, float* obuf, int ld_o, hipStream_t s);
+bool retention_chunk_supported(int D, int Dv);
 
 struct MoeParams {
   const float* proj;    // [B][ld]: router logits at off_router, shared: scalar gate, gate rows, up rows
@@ -106,7 +110,27 @@ struct MoeParams {
 void moe_route(const MoeParams& P, hipStream_t s);   // top-k ids + softmax weights, shared gate and activation
 void moe_experts(const MoeParams& P, hipStream_t s); // gate/up + activation of the routed experts -> hmid
 void moe_down(const MoeParams& P, hipStream_t s);    // y = sum_j w_j down_j(hmid_j) + sgate * shared_down(hmid_s)
+// a few rows (decode steps): routing + routed and shared activations in one launch, then the experts' down
+// projections, the mixer's output projection (a [B][lda] . w_o [E][Ko]) and the residual update
+// x += mult * (...) in a second one
+void moe_fused_small(const MoeParams& P, const void* a, int lda, const void* w_o, int Ko, float* x, float mult,
+                     hipStream_t s);
 constexpr int MOE_MAX_TOP = 16;
+// prompt portions (bfloat16): after moe_route, the (row, expert) pairs are sorted by expert and every expert's
+// rows go through the matrix-core product together; y as moe_down leaves it
+struct MoeGroupWs {
+  int* rank;     // [max_pairs]
+  int* srow;     // [max_pairs] sorted position -> pair
+  int* inv;      // [max_pairs] pair -> sorted position
+  int* tiles;    // [max_tiles][3]
+  int* ntiles;   // [1]
+  float* gu;     // [max_pairs][2F]
+  void* hs;      // [max_pairs][F] matrix dtype
+  float* ds;     // [max_pairs][E]
+  int max_pairs, max_tiles;
+};
+void moe_grouped(const MoeParams& P, const MoeGroupWs& W, hipStream_t s);
+bool moe_grouped_supported(const MoeParams& P);
 
 }  // namespace stack
 }  // namespace omx

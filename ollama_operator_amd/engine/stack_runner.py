@@ -62,7 +62,8 @@ class StackExec:
         e.set_workspace(dict(resid=p(r.resid), x0=p(r.x0), h=p(r.hbuf), cat=p(r.catbuf), proj=p(r.proj),
                              ld_proj=r.proj.shape[1], a=p(r.abuf), ld_a=r.abuf.shape[1], hmid=p(r.hmid),
                              ld_hmid=r.hmid.shape[1], y=p(r.ybuf), eids=p(r.eids), ew=p(r.ew), ld_top=r.eids.shape[1],
-                             sgate=p(r.sgate), lrows=p(r.lbuf)))
+                             sgate=p(r.sgate), lrows=p(r.lbuf), obuf=p(r.obuf), ld_obuf=r.obuf.shape[1],
+                             **{"moe_" + k: (v if isinstance(v, int) else p(v)) for k, v in r.moe_ws.items()}))
         e.set_inputs(dict(tokens=p(r.d_tokens), pos=p(r.d_pos), slot=p(r.d_slot), q_len=p(r.d_qlen),
                           q_seq=p(r.d_qseq), block_table=p(r.d_block_table), max_blocks=r.max_blocks,
                           bs=r.block_size, logits=p(r.logits), ld_logits=r.logits.shape[1],
@@ -126,7 +127,17 @@ class StackRunner(Runner):
         self.ew = torch.zeros(max_batch, top, **f32)
         self.sgate = torch.zeros(max_batch, **f32)
         self.lbuf = torch.zeros(max_batch, E, **tt)
-        self.ext, self._ext_map, self._ext_next = None, {}, 0
+        self.obuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **f32)  # retention, before its norm
+        # routed feed-forward of prompt portions (bfloat16): pairs sorted by expert, per-expert matrix-core products
+        self.moe_ws = {}
+        if mlps and T == torch.bfloat16:
+            pairs = max_batch * top
+            tiles = pairs // 64 + max(f.experts for f in mlps) + 1
+            self.moe_ws = dict(rank=torch.zeros(pairs, **i32), srow=torch.zeros(pairs, **i32), inv=torch.zeros(pairs, **i32),
+                               tiles=torch.zeros(3 * tiles, **i32), ntiles=torch.zeros(1, **i32),
+                               gu=torch.zeros(pairs, 2 * max(f.ff for f in mlps), **f32),
+                               hs=torch.zeros(pairs, max(f.ff for f in mlps), **tt), ds=torch.zeros(pairs, E, **f32),
+                               max_pairs=pairs, max_tiles=tiles)
         self.mfma_bytes = self.lib_min = self.moe_lib = 0
         self.w16 = self.mb_bufs = self.x8_bufs = None
         self._alloc_step_state(V, n_blocks)
@@ -187,6 +198,20 @@ class StackRunner(Runner):
                 raise RuntimeError(f"sequence {sid}: a recurrent state cannot be cut back from {s.length} to {keep}")
             self._clear_slot(s.row)
         super()._keep_prefix(sid, keep, history)
+
+    def _graph(self, B: int, steps: int = 1, inst: int = 0):
+        """A graph captured in mid-generation: the warm-up forward that precedes the capture really runs, and a
+        second run of the same rows would advance their recurrent states twice (a K/V write is the same write
+        again, a state update is not). The states are put back after it."""
+        key = (B, self._decode_S, steps, inst)
+        if key in self.graphs:
+            return self.graphs[key]
+        saved = [st.clone() if st is not None else None for st in self.states]
+        g = super()._graph(B, steps, inst)
+        for st, old in zip(self.states, saved):
+            if st is not None:
+                st.copy_(old)
+        return g
 
     # ------------------------------------------------------------------ load-time warm-up
     def warmup(self) -> None:

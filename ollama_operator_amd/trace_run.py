@@ -30,6 +30,7 @@ def _ensure_built(stack: bool) -> None:
     """A fresh checkout has no built library: compile what this model's engine needs, and only that."""
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     sys.path.insert(0, root)
+    import torch  # noqa: F401  (first: the native modules share the HIP runtime that torch ships)
     import build_native
     if stack:
         try:
