@@ -48,6 +48,8 @@ PYBIND11_MODULE(_stack, m) {
   m.def("gemm_path", &gemm_path);
   m.def("set_gemm_mfma", &set_gemm_mfma);
   m.def("retention_supported", &retention_supported);
+  m.def("retention_chunk_rows", &retention_chunk_rows);
+  m.attr("FLASH_TILE_ROWS") = (int)FLASH_TILE_ROWS;
 
   py::class_<StackExecutor>(m, "Executor")
       .def(py::init<>())
@@ -138,7 +140,12 @@ PYBIND11_MODULE(_stack, m) {
         w.ld_top = geti(d, "ld_top");
         w.sgate = Pp<float>(ptr(d, "sgate"));
         w.lrows = Pp<void>(ptr(d, "lrows"));
-        w.obuf = Pp<float>(ptr(d, "obuf"));
+        w.ret.chunks = Pp<const int>(ptr(d, "ret_chunks"));
+        w.ret.max_chunks = geti(d, "ret_max_chunks");
+        w.ret.U = Pp<float>(ptr(d, "ret_u"));
+        w.ret.Sin = Pp<float>(ptr(d, "ret_sin"));
+        w.ret.u_stride = d.contains("ret_u_stride") ? d["ret_u_stride"].cast<long long>() : 0;
+        w.ret.obuf = Pp<float>(ptr(d, "obuf"));
         w.moe.rank = Pp<int>(ptr(d, "moe_rank"));
         w.moe.srow = Pp<int>(ptr(d, "moe_srow"));
         w.moe.inv = Pp<int>(ptr(d, "moe_inv"));
@@ -149,7 +156,7 @@ PYBIND11_MODULE(_stack, m) {
         w.moe.ds = Pp<float>(ptr(d, "moe_ds"));
         w.moe.max_pairs = geti(d, "moe_max_pairs");
         w.moe.max_tiles = geti(d, "moe_max_tiles");
-        w.ld_obuf = geti(d, "ld_obuf");
+        w.ret.ld_o = geti(d, "ld_obuf");
       })
       .def("set_inputs", [](StackExecutor& e, py::dict d) {
         StackInputs& in = e.in;
@@ -166,6 +173,18 @@ PYBIND11_MODULE(_stack, m) {
         in.logit_idx = Pp<const int>(ptr(d, "logit_idx"));
         if (in.bs <= 0 || in.max_blocks <= 0) throw std::runtime_error("bad block geometry");
         e.validate();
+      })
+      .def("bind_tiles", [](StackExecutor& e, uintptr_t table, int max_tiles) {
+        e.tiles = Pp<const int>(table);
+        e.max_tiles = max_tiles;
+      })
+      .def("set_tiles", [](StackExecutor& e, int n) {
+        if (n < 0 || n > e.max_tiles) throw std::runtime_error("stack executor: tile count outside the table");
+        e.n_tiles = n;
+      })
+      .def("set_chunks", [](StackExecutor& e, int n) {
+        if (n < 0 || n > e.ws.ret.max_chunks) throw std::runtime_error("stack executor: chunk count outside the table");
+        e.n_chunks = n;
       })
       .def("step", [](StackExecutor& e, int stage, int idx, int B, int n_logits, bool use_idx, uintptr_t stream) {
         if (B <= 0 || B > e.cfg.max_B || n_logits < 0 || n_logits > e.cfg.max_B)

@@ -51,24 +51,35 @@ void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
     GemmParams g{ws.cat, 2 * E, loop_in, B, E, 2 * E, ws.resid, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
     gemm(g, s);
   }
-  layer_norm_cast(ws.resid, nullptr, B, E, L.norm_w, L.norm_b, cfg.eps, ws.h, f32, s);
-  {  // every matrix that reads the normed activations, in one product
+  StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
+  AttnParams A{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.softcap,
+               L.qtemp_coef, L.qtemp_every, r.kc, r.vc, ws.a, ws.ld_a, f32};
+  const bool fused_in = gemv_ln_supported(B, E, f32);
+  if (fused_in) {  // decode steps: norm + input projection (+ query temperature and K/V store) in one launch
+    gemv_ln(ws.resid, E, L.norm_w, L.norm_b, cfg.eps, L.w_in, B, L.n_in, ws.proj, ws.ld_proj, ws.h, L.kind == 0 ? &A : nullptr,
+            &R, f32, s);
+  } else {
+    layer_norm_cast(ws.resid, nullptr, B, E, L.norm_w, L.norm_b, cfg.eps, ws.h, f32, s);
+    // every matrix that reads the normed activations, in one product
     GemmParams g{ws.h, E, L.w_in, B, L.n_in, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
     gemm(g, s);
   }
-  StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
   if (L.kind == 0) {
-    AttnParams A{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.softcap,
-                 L.qtemp_coef, L.qtemp_every, r.kc, r.vc, ws.a, ws.ld_a, f32};
-    attn_prepare(A, R, s);
-    attention(A, R, s);
+    if (!fused_in) attn_prepare(A, R, s);
+    if (B > SMALL_B && n_tiles > 0 && tiles && flash_prefill_supported(A))
+      flash_prefill(A, R, tiles, n_tiles, s);  // prompt portions: query tiles on the matrix cores
+    else
+      attention(A, R, s);
   } else {
     RetParams P{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.off_g, L.heads, L.dim, L.vdim, L.rot_dims, L.inv_freq,
                 L.decay, r.state, cfg.eps, ws.a, ws.ld_a, f32};
-    // prompt portions in chunks; a few rows (decode steps) token by token in one launch
-    if (B > SMALL_B && ws.obuf && ws.ld_obuf >= L.heads * L.vdim && retention_chunk_supported(L.dim, L.vdim))
-      retention_chunked(P, R, ws.obuf, ws.ld_obuf, s);
-    else
+    // prompt portions in chunks (the host bound this step's chunk table); else token by token in one launch
+    if (B > SMALL_B && n_chunks > 0 && ws.ret.U && ws.ret.ld_o >= L.heads * L.vdim &&
+        ws.ret.u_stride >= (long long)L.heads * L.dim * L.vdim && retention_chunk_supported(L.dim, L.vdim)) {
+      RetChunkWs W = ws.ret;
+      W.nchunks = n_chunks;
+      retention_chunked(P, R, W, s);
+    } else
       retention(P, R, s);
   }
   const float* ff = nullptr;

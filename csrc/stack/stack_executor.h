@@ -64,8 +64,7 @@ struct StackWorkspace {
   float* sgate = nullptr;
   void* lrows = nullptr;   // [max_B][E] matrix dtype: normed rows for the head
   MoeGroupWs moe{};        // grouped routed feed-forward (prompt portions, bfloat16); gu == null: unused
-  float* obuf = nullptr;   // [max_B][ld_obuf] float32: retention outputs before their norm (chunked path)
-  int ld_obuf = 0;
+  RetChunkWs ret{};        // chunked retention (prompt portions): chunk table, per-chunk states, o before its norm
 };
 
 struct StackInputs {
@@ -95,6 +94,9 @@ class StackExecutor {
   const void* head_w = nullptr;
   StackWorkspace ws;
   StackInputs in;
+  const int* tiles = nullptr;  // attention query tiles of the NEXT step {first row, rows}, n_tiles of them (0: none)
+  int n_tiles = 0, max_tiles = 0;
+  int n_chunks = 0;        // chunks in ws.ret.chunks for the NEXT step (0: none bound, retention runs token by token)
 
   void validate() const;  // throws when a size does not fit the kernels or a pointer is missing
   void embed(int B, hipStream_t s);

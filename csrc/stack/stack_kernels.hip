@@ -141,6 +141,92 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const T* __restrict__ A,
   }
 }
 
+// ---- decode steps: layer norm + input projection (+ the attention layer's query temperature and K/V store)
+// Every block normalises the step's few rows again (they are E floats each) into LDS, rounded to the matrix
+// dtype as the unfused path stores them, then its four waves take one weight row each. Block 0 also writes the
+// normed rows out for the routed experts. QkvEpi: outputs in the q range are multiplied by the row's query
+// temperature, outputs in the k and v ranges are also stored at the row's cache slot.
+struct QkvEpi {
+  int on;
+  int off_q, n_q, off_k, n_k, off_v, n_v;
+  int G, D, Dv, bs;
+  float coef;
+  int every;
+  const int* pos;
+  const int* slot;
+  void* kc;
+  void* vc;
+};
+constexpr int LN_LDS_BYTES = 32768;
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ x, int E, const float* __restrict__ nw,
+                                                      const float* __restrict__ nb, float eps, const T* __restrict__ W,
+                                                      int M, int N, float* __restrict__ C, int ldc, T* __restrict__ hout,
+                                                      QkvEpi q, int vec) {
+  __shared__ __attribute__((aligned(16))) unsigned char hs_raw[LN_LDS_BYTES];
+  __shared__ float red[4];
+  T* hs = (T*)hs_raw;
+  const int tid = threadIdx.x, lane = tid & 63;
+  for (int m = 0; m < M; ++m) {
+    const float* row = x + (long long)m * E;
+    float sum = 0.f;
+    for (int i = tid; i < E; i += 256) sum += row[i];
+    const float mean = block_sum256(sum, red) / (float)E;
+    float sq = 0.f;
+    for (int i = tid; i < E; i += 256) {
+      const float d = row[i] - mean;
+      sq += d * d;
+    }
+    const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)E + eps);
+    for (int i = tid; i < E; i += 256) {
+      st(hs + (long long)m * E + i, (row[i] - mean) * rstd * nw[i] + nb[i]);
+      if (blockIdx.x == 0) hout[(long long)m * E + i] = hs[(long long)m * E + i];
+    }
+  }
+  __syncthreads();
+  const int n = blockIdx.x * 4 + (tid >> 6);
+  if (n >= N) return;
+  const T* w = W + (long long)n * E;
+  for (int m = 0; m < M; ++m) {
+    float acc = wave_dot<T>(w, hs + (long long)m * E, E, lane, vec != 0);
+    if (lane == 0) {
+      if (q.on) {
+        if (n >= q.off_q && n < q.off_q + q.n_q) {
+          if (q.coef != 0.f) acc *= 1.f + q.coef * logf(floorf((float)(q.pos[m] + 1) / (float)q.every) + 1.f);
+        } else if (n >= q.off_k && n < q.off_k + q.n_k) {
+          const int i = n - q.off_k, slot = q.slot[m];
+          const long long blk = slot / q.bs, off = slot % q.bs;
+          st((T*)q.kc + ((blk * q.G + i / q.D) * q.bs + off) * q.D + i % q.D, acc);
+        } else if (n >= q.off_v && n < q.off_v + q.n_v) {
+          const int i = n - q.off_v, slot = q.slot[m];
+          const long long blk = slot / q.bs, off = slot % q.bs;
+          st((T*)q.vc + ((blk * q.G + i / q.Dv) * q.bs + off) * q.Dv + i % q.Dv, acc);
+        }
+      }
+      C[(long long)m * ldc + n] = acc;
+    }
+  }
+}
+bool gemv_ln_supported(int M, int E, int f32) { return M > 0 && M <= 8 && (long long)M * E * (f32 ? 4 : 2) <= LN_LDS_BYTES; }
+void gemv_ln(const float* x, int E, const float* nw, const float* nb, float eps, const void* W, int M, int N, float* C,
+             int ldc, void* hout, const AttnParams* A, const StepRows* R, int f32, hipStream_t s) {
+  check(gemv_ln_supported(M, E, f32) && x && nw && nb && W && C && hout && N > 0 && ldc >= N, "gemv_ln: bad operands");
+  QkvEpi q{};
+  if (A) {
+    check(R && R->pos && R->slot && A->kc && A->vc, "gemv_ln: attention epilogue without rows or pools");
+    q = QkvEpi{1, A->off_q, A->H * A->D, A->off_k, A->G * A->D, A->off_v, A->G * A->Dv, A->G, A->D, A->Dv, R->bs,
+               A->qtemp_coef, A->qtemp_every, R->pos, R->slot, A->kc, A->vc};
+  }
+  dim3 grid((N + 3) / 4);
+  if (f32)
+    hipLaunchKernelGGL(gemv_ln_kernel<float>, grid, dim3(256), 0, s, x, E, nw, nb, eps, (const float*)W, M, N, C, ldc,
+                       (float*)hout, q, (int)(E % 4 == 0 && ((uintptr_t)W & 15) == 0));
+  else
+    hipLaunchKernelGGL(gemv_ln_kernel<bf16>, grid, dim3(256), 0, s, x, E, nw, nb, eps, (const bf16*)W, M, N, C, ldc,
+                       (bf16*)hout, q, (int)(E % 8 == 0 && ((uintptr_t)W & 15) == 0));
+  launched("gemv_ln");
+}
+
 // ------------------------------------------------------------------------------------------------ FMA tile GEMM
 // 64 x 64 output tile per block, K in steps of 16 through LDS, 4 x 4 outputs per thread; true float32
 template <typename T>
@@ -516,14 +602,21 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
       rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
       const T* kr = kc + (long long)rowidx * P.D;
       if (vec) {
-        for (int d = 0; d < P.D; d += 8) {
-          float k8[8];
-          load8<T>(kr + d, k8);
+        for (int d0 = 0; d0 < P.D; d0 += 64) {  // 64 dims of the row in flight at a time
+          float k8[8][8];
 #pragma unroll
-          for (int r = 0; r < RQ; ++r) {
-            const f32x4 qa = *(const f32x4*)&qs[qw][r][d], qb = *(const f32x4*)&qs[qw][r][d + 4];
-            dot[r] += qa[0] * k8[0] + qa[1] * k8[1] + qa[2] * k8[2] + qa[3] * k8[3] + qb[0] * k8[4] + qb[1] * k8[5] +
-                      qb[2] * k8[6] + qb[3] * k8[7];
+          for (int u = 0; u < 8; ++u) load8<T>(kr + min(d0 + 8 * u, P.D - 8), k8[u]);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int d = d0 + 8 * u;
+            if (d < P.D) {
+#pragma unroll
+              for (int r = 0; r < RQ; ++r) {
+                const f32x4 qa = *(const f32x4*)&qs[qw][r][d], qb = *(const f32x4*)&qs[qw][r][d + 4];
+                dot[r] += qa[0] * k8[u][0] + qa[1] * k8[u][1] + qa[2] * k8[u][2] + qa[3] * k8[u][3] + qb[0] * k8[u][4] +
+                          qb[1] * k8[u][5] + qb[2] * k8[u][6] + qb[3] * k8[u][7];
+              }
+            }
           }
         }
       } else {
@@ -550,19 +643,20 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
       for (int c = 0; c < DC; ++c) acc[r][c] *= corr;
       m[r] = mn;
     }
-    // values: 8 keys' rows in flight at a time (a key past the group's end reads row 0 with weight 0)
+    // values: UB keys' rows in flight at a time (a key past the group's end reads row 0 with weight 0)
+    constexpr int UB = 32 / DC;
     const int cnt = min(64, n - t0);
-    for (int j0 = 0; j0 < cnt; j0 += 8) {
-      float v[8][DC];
+    for (int j0 = 0; j0 < cnt; j0 += UB) {
+      float v[UB][DC];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < UB; ++u) {
         const int rj = __shfl(rowidx, j0 + u, 64);
         const T* vr = vc + (long long)rj * P.Dv;
 #pragma unroll
         for (int c = 0; c < DC; ++c) v[u][c] = (lane + 64 * c < P.Dv) ? ld(vr + lane + 64 * c) : 0.f;
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < UB; ++u)
 #pragma unroll
         for (int r = 0; r < RQ; ++r) {
           const float pj = __shfl(p[r], j0 + u, 64);  // 0 for keys past the end
@@ -642,6 +736,181 @@ static void launch_attention(const AttnParams& P, const StepRows& R, hipStream_t
   else
     launch_attention_r<T, 1>(P, R, nbatch, vec, s);
 }
+// ---- prompt portions on the matrix cores (bfloat16 K/V pools). One wave per (tile of up to 32 query rows of one
+// sequence, query head); the host lists the tiles {first row, rows}. Keys go by 32 at a time:
+//   S^T[key][q] = K Q^T      v_mfma_f32_32x32x16_bf16, A = K rows read straight from the pool (16-byte pieces),
+//                            B = the tile's queries, kept in registers as bf16 high + low parts (two products,
+//                            so the float32 queries keep ~16 bits of mantissa);
+//   scale, cap, mask, running maximum and sum per query: lane (q, half) holds 16 keys of ITS query, so the
+//                            softmax statistics are per-lane values plus one exchange between the two halves;
+//   O^T[dv][q] += V^T P^T    A = V^T gathered from the wave's LDS copy of the 32 V rows, B = the weights, again
+//                            as high + low bf16 parts; O^T keeps each lane's query in the lane, so the running
+//                            rescale is a per-lane multiply.
+// The K operand rows are loaded in the order key(m) = m with bits 2 and 3 swapped: the accumulator registers
+// 0..7 / 8..15 of lane (q, half) then hold keys 8 half + 0..7 of the first / second 16-key group, which is the
+// operand layout of the second product, so the weights never move between lanes.
+constexpr int FL_LDV = 4;  // LDS row padding (elements): the two lane halves land in different banks
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pack_bf(float a, float b) {  // round to nearest even (v_cvt_pk_bf16_f32)
+  const bf16x2 v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(unsigned, v);
+}
+// float32 exp and tanh on the transcendental unit (v_exp_f32, 1 ulp): the error stays below 1e-6 of the cap
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = __builtin_amdgcn_exp2f(fminf(x, 15.f) * 2.88539008177792681f);  // e^(2x)
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+template <int KD, int NV>
+__global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRows R, const int* __restrict__ tiles) {
+  constexpr int D = 16 * KD, DV = 32 * NV, LDV = DV + FL_LDV;
+  __shared__ __attribute__((aligned(16))) uint16_t Vl[32 * LDV];
+  const int lane = threadIdx.x, q = lane & 31, hf = lane >> 5;
+  const int row0 = tiles[2 * blockIdx.x], nrows = tiles[2 * blockIdx.x + 1];
+  const int h = blockIdx.y, g = h / (P.H / P.G);
+  const int* bt = R.block_table + (long long)R.q_seq[row0] * R.max_blocks;
+  const int qrow = row0 + min(q, nrows - 1);
+  const int qlen = q < nrows ? R.q_len[qrow] : 0;
+  const int kmax = R.q_len[row0 + nrows - 1];
+  // queries: B operand, lane (q, hf) holds dims 16 kk + 8 hf + 0..7
+  bf16x8 qhi[KD], qlo[KD];
+  {
+    const float* qp = P.proj + (long long)qrow * P.ld + P.off_q + h * D + 8 * hf;
+#pragma unroll
+    for (int kk = 0; kk < KD; ++kk) {
+      const f32x4 a = *(const f32x4*)(qp + 16 * kk), b = *(const f32x4*)(qp + 16 * kk + 4);
+      const float x[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+      u32x4 hi, lo;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        hi[i] = pack_bf(x[2 * i], x[2 * i + 1]);
+        lo[i] = pack_bf(x[2 * i] - __uint_as_float(hi[i] << 16), x[2 * i + 1] - __uint_as_float(hi[i] & 0xffff0000u));
+      }
+      qhi[kk] = __builtin_bit_cast(bf16x8, hi);
+      qlo[kk] = __builtin_bit_cast(bf16x8, lo);
+    }
+  }
+  const int m = lane & 31;
+  const int kperm = (m & 0x13) | ((m & 4) << 1) | ((m & 8) >> 1);  // bits 2 and 3 swapped
+  f32x16 o[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[j][r] = 0.f;
+  float mi = -1e30f, li = 0.f;
+  const float inv_cap = P.softcap != 0.f ? 1.f / P.softcap : 0.f;
+  const uint16_t* kc = (const uint16_t*)P.kc;
+  const uint16_t* vc = (const uint16_t*)P.vc;
+  for (int t0 = 0; t0 < kmax; t0 += 32) {
+    // V rows of this key group into LDS (keys past the end: the last key's row, their weights are zero)
+    __syncthreads();
+    {
+      constexpr int CH = DV / 8;  // 16-byte pieces per row
+#pragma unroll
+      for (int c = lane; c < 32 * CH; c += 64) {
+        const int key = min(t0 + c / CH, kmax - 1), seg = c % CH;
+        const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
+        const u32x4 v = *(const u32x4*)(vc + rowidx * DV + 8 * seg);
+        unsigned* dst = (unsigned*)&Vl[(c / CH) * LDV + 8 * seg];
+        *(unsigned long long*)dst = (unsigned long long)v[0] | ((unsigned long long)v[1] << 32);
+        *(unsigned long long*)(dst + 2) = (unsigned long long)v[2] | ((unsigned long long)v[3] << 32);
+      }
+    }
+    // S^T = K Q^T
+    f32x16 sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    {
+      const int key = min(t0 + kperm, kmax - 1);
+      const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
+      const uint16_t* kr = kc + rowidx * D + 8 * hf;
+#pragma unroll
+      for (int kk = 0; kk < KD; ++kk) {
+        const bf16x8 kf = __builtin_bit_cast(bf16x8, *(const u32x4*)(kr + 16 * kk));
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qhi[kk], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qlo[kk], sacc, 0, 0, 0);
+      }
+    }
+    // register r of lane (q, hf) is key t0 + 16 (r >> 3) + 8 hf + (r & 7)
+    float pr[16];
+    float mx = -1e30f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float sc = sacc[r] * P.scale;
+      if (P.softcap != 0.f) sc = P.softcap * fast_tanh(sc * inv_cap);
+      const bool vis = t0 + 16 * (r >> 3) + 8 * hf + (r & 7) < qlen;
+      pr[r] = vis ? sc : -1e30f;
+      mx = fmaxf(mx, pr[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(mi, mx);
+    const float corr = fast_exp(fmaxf(mi - mn, -100.f));
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      pr[r] = pr[r] > -1e29f ? fast_exp(pr[r] - mn) : 0.f;
+      sum += pr[r];
+    }
+    sum += __shfl_xor(sum, 32, 64);
+    li = li * corr + sum;
+    mi = mn;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[j][r] *= corr;
+    bf16x8 phi[2], plo[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      u32x4 hi, lo;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a = pr[8 * ks + 2 * i], b = pr[8 * ks + 2 * i + 1];
+        hi[i] = pack_bf(a, b);
+        lo[i] = pack_bf(a - __uint_as_float(hi[i] << 16), b - __uint_as_float(hi[i] & 0xffff0000u));
+      }
+      phi[ks] = __builtin_bit_cast(bf16x8, hi);
+      plo[ks] = __builtin_bit_cast(bf16x8, lo);
+    }
+    __syncthreads();  // the V rows are in LDS
+    // O^T += V^T P^T: A operand lane (dv = 32 j + m, hf) holds V[16 ks + 8 hf + i][dv], i = 0..7
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const uint16_t* vp = &Vl[(16 * ks + 8 * hf) * LDV + 32 * j + m];
+        u32x4 vv;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vv[i] = (unsigned)vp[(2 * i) * LDV] | ((unsigned)vp[(2 * i + 1) * LDV] << 16);
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, vv);
+        o[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, phi[ks], o[j], 0, 0, 0);
+        o[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, plo[ks], o[j], 0, 0, 0);
+      }
+  }
+  if (q < nrows) {  // register r of tile j: value dim 32 j + (r & 3) + 8 (r >> 2) + 4 hf of this lane's query
+    bf16* out = (bf16*)P.out + (long long)qrow * P.ld_out + h * DV;
+    const float inv = 1.f / li;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st(out + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hf, o[j][r] * inv);
+  }
+}
+bool flash_prefill_supported(const AttnParams& P) {
+  return !P.f32 && P.D == P.Dv && (P.D == 64 || P.D == 96 || P.D == 128) && P.ld % 4 == 0 && P.off_q % 4 == 0 &&
+         ((uintptr_t)P.proj & 15) == 0 && ((uintptr_t)P.kc & 15) == 0 && ((uintptr_t)P.vc & 15) == 0;
+}
+void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s) {
+  check(flash_prefill_supported(P) && tiles && ntiles > 0 && P.G > 0 && P.H % P.G == 0 && P.out, "flash prefill: operands");
+  dim3 grid(ntiles, P.H);
+  if (P.D == 64)
+    hipLaunchKernelGGL((flash_prefill_kernel<4, 2>), grid, dim3(64), 0, s, P, R, tiles);
+  else if (P.D == 96)
+    hipLaunchKernelGGL((flash_prefill_kernel<6, 3>), grid, dim3(64), 0, s, P, R, tiles);
+  else
+    hipLaunchKernelGGL((flash_prefill_kernel<8, 4>), grid, dim3(64), 0, s, P, R, tiles);
+  launched("flash_prefill");
+}
+
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && P.out,
         "attention: head sizes up to 256, heads a multiple of key/value heads");
@@ -731,129 +1000,164 @@ __global__ __launch_bounds__(256) void retention_kernel(RetParams P, StepRows R)
     if (act && i < D) st_base[(long long)i * Dv + j] = S[ii];
   }
 }
-// Prompt portions: the same recurrence in chunks of RC tokens. With g the head's decay, a chunk that starts
-// from state S computes, for its tokens t, s = 0 .. n - 1,
+// Prompt portions: the same recurrence in chunks of RC tokens. With g the head's decay, a chunk of n tokens that
+// starts from state S computes, for its tokens t, s = 0 .. n - 1,
 //   A[t][s] = (q_t . k_s) g^(t - s) for s <= t,   o_t = g^(t + 1) S^T q_t + sum_s A[t][s] v_s,
-//   S <- g^n S + sum_s g^(n - 1 - s) k_s v_s^T,
-// all in float32 on the vector ALUs. One block per (segment, head, 64 value columns): thread (g4, j) keeps
-// column j of S in registers, produces o_t[j] for t = g4, g4 + 4, ..., and the four threads of a column advance
-// their copies of it alike. The un-normalised o goes to `obuf`; retention_finish_kernel applies the per-head
-// unit RMS and the gate.
+//   U = sum_s g^(n - 1 - s) k_s v_s^T,             S <- g^n S + U,
+// all in float32 on the vector ALUs, in three launches over a host-built chunk table {first row, rows, state
+// slot, flags (1: first chunk of its sequence's rows, 2: last)}:
+//   1. every chunk's U, chunks in parallel                      (retention_u_kernel)
+//   2. the scan S <- g^n S + U over each sequence's chunks, one thread per state element, which leaves every
+//      chunk's incoming state and the sequence's final state    (retention_scan_kernel)
+//   3. every chunk's outputs from its incoming state, in parallel (retention_out_kernel)
+// then retention_finish_kernel applies the per-head unit RMS and the gate.
+// Blocks of 1. and 3. take (chunk, head, 64 value columns); thread (g4, j) = (tid / 64, tid % 64).
 constexpr int RC = 32;
+// rotated q and scaled rotated k of the chunk's rows into LDS (rows past n and dims past D zero)
+template <int MAXD, bool WITH_Q>
+__device__ __forceinline__ void stage_qk(const RetParams& P, const StepRows& R, int row0, int cn, int h,
+                                         float (*Qs)[MAXD], float (*Ks)[MAXD + 4]) {
+  const int D = P.D, half = P.rot_dims / 2, tid = threadIdx.x;
+  const float kscale = 1.f / sqrtf((float)D);
+  constexpr int IT = RC * MAXD / 256;
+  float qa[IT], qb[IT], ka[IT], kb[IT], ang[IT];
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {  // every load first: one round trip for the chunk
+    const int idx = tid + 256 * it;
+    const int c = idx / MAXD, d = idx % MAXD;
+    qa[it] = qb[it] = ka[it] = kb[it] = ang[it] = 0.f;
+    if (c < cn && d < D) {
+      const int r = row0 + c;
+      const float* q = P.proj + (long long)r * P.ld + P.off_q + h * D;
+      const float* k = P.proj + (long long)r * P.ld + P.off_k + h * D;
+      ka[it] = k[d];
+      if (WITH_Q) qa[it] = q[d];
+      if (d < P.rot_dims) {
+        const int pd = d < half ? d + half : d - half;
+        kb[it] = k[pd];
+        if (WITH_Q) qb[it] = q[pd];
+        ang[it] = (float)R.pos[r] * P.inv_freq[d < half ? d : d - half];
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + 256 * it;
+    const int c = idx / MAXD, d = idx % MAXD;
+    float qv = qa[it], kv = ka[it];
+    if (c < cn && d < P.rot_dims) {  // (u, v) -> (u cos - v sin, v cos + u sin), u the lower dim of the pair
+      const float cs = cosf(ang[it]), sn = sinf(ang[it]);
+      const float sg = d < half ? -1.f : 1.f;
+      qv = qa[it] * cs + sg * qb[it] * sn;
+      kv = ka[it] * cs + sg * kb[it] * sn;
+    }
+    if (WITH_Q) Qs[c][d] = qv;
+    Ks[c][d] = kv * kscale;
+  }
+}
+__device__ __forceinline__ void stage_v(const RetParams& P, int row0, int cn, int h, int jb, float (*Vs)[64]) {
+  for (int idx = threadIdx.x; idx < RC * 64; idx += 256) {
+    const int c = idx >> 6, jj = idx & 63;
+    const int cc = jb * 64 + jj;
+    Vs[c][jj] = (c < cn && cc < P.Dv) ? P.proj[(long long)(row0 + c) * P.ld + P.off_v + h * P.Dv + cc] : 0.f;
+  }
+}
 template <int MAXD>
-__global__ __launch_bounds__(256) void retention_chunk_kernel(RetParams P, StepRows R, float* __restrict__ obuf,
-                                                              int ld_o, int NJ) {
+__global__ __launch_bounds__(256) void retention_u_kernel(RetParams P, StepRows R, const int* __restrict__ chunks,
+                                                          float* __restrict__ U, long long u_stride, int NJ) {
+  __shared__ __attribute__((aligned(16))) float Ks[RC][MAXD + 4];
+  __shared__ float Vs[RC][64];
+  __shared__ float pw[RC + 1];
+  const int c = blockIdx.x, h = blockIdx.y / NJ, jb = blockIdx.y % NJ, tid = threadIdx.x;
+  const int row0 = chunks[4 * c], cn = chunks[4 * c + 1];
+  const int j = tid & 63, g4 = tid >> 6, col = jb * 64 + j;
+  if (tid <= RC) pw[tid] = powf(P.decay[h], (float)tid);
+  stage_qk<MAXD, false>(P, R, row0, cn, h, nullptr, Ks);
+  stage_v(P, row0, cn, h, jb, Vs);
+  __syncthreads();
+  float u[MAXD / 4];
+#pragma unroll
+  for (int ii = 0; ii < MAXD / 4; ++ii) u[ii] = 0.f;
+  for (int sx = 0; sx < cn; ++sx) {
+    const float vv = Vs[sx][j] * pw[cn - 1 - sx];
+#pragma unroll
+    for (int ii = 0; ii < MAXD / 4; ++ii) u[ii] += Ks[sx][g4 + 4 * ii] * vv;
+  }
+  if (col < P.Dv) {
+    float* out = U + c * u_stride + (long long)h * P.D * P.Dv;
+#pragma unroll
+    for (int ii = 0; ii < MAXD / 4; ++ii) {
+      const int i = g4 + 4 * ii;
+      if (i < P.D) out[(long long)i * P.Dv + col] = u[ii];
+    }
+  }
+}
+__global__ __launch_bounds__(256) void retention_scan_kernel(RetParams P, const int* __restrict__ chunks, int nchunks,
+                                                             const float* __restrict__ U, float* __restrict__ Sin,
+                                                             long long u_stride) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long per_head = (long long)P.D * P.Dv;
+  if (e >= P.H * per_head) return;
+  const float dec = P.decay[e / per_head];
+  const float dfull = powf(dec, (float)RC);
+  float S = 0.f;
+  for (int c = 0; c < nchunks; ++c) {
+    const int cn = chunks[4 * c + 1], slot = chunks[4 * c + 2], flags = chunks[4 * c + 3];
+    float* st_e = P.state + (long long)slot * P.H * per_head + e;
+    if (flags & 1) S = *st_e;
+    Sin[c * u_stride + e] = S;
+    S = (cn == RC ? dfull : powf(dec, (float)cn)) * S + U[c * u_stride + e];
+    if (flags & 2) *st_e = S;
+  }
+}
+template <int MAXD>
+__global__ __launch_bounds__(256) void retention_out_kernel(RetParams P, StepRows R, const int* __restrict__ chunks,
+                                                            const float* __restrict__ Sin, long long u_stride,
+                                                            float* __restrict__ obuf, int ld_o, int NJ) {
   __shared__ __attribute__((aligned(16))) float Qs[RC][MAXD];
   __shared__ __attribute__((aligned(16))) float Ks[RC][MAXD + 4];
   __shared__ float Vs[RC][64];
   __shared__ float As[RC][RC + 1];
   __shared__ float pw[RC + 1];
-  __shared__ int seg_n;
-  const int r0 = blockIdx.x, h = blockIdx.y / NJ, jb = blockIdx.y % NJ, tid = threadIdx.x;
-  const int seq = R.q_seq[r0];
-  if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;
+  const int c = blockIdx.x, h = blockIdx.y / NJ, jb = blockIdx.y % NJ, tid = threadIdx.x;
+  const int row0 = chunks[4 * c], cn = chunks[4 * c + 1];
   const int D = P.D, Dv = P.Dv;
-  const int j = tid & 63, g4 = tid >> 6;
-  const int col = jb * 64 + j;
+  const int j = tid & 63, g4 = tid >> 6, col = jb * 64 + j;
   const bool colok = col < Dv;
-  const float dec = P.decay[h];
-  if (tid == 0) seg_n = R.B - r0;
-  if (tid <= RC) pw[tid] = powf(dec, (float)tid);
-  __syncthreads();
-  for (int i = 1 + tid; r0 + i < R.B; i += 256)  // the segment ends at the first row of another sequence
-    if (R.q_seq[r0 + i] != seq) {
-      atomicMin(&seg_n, i);
-      break;
-    }
+  if (tid <= RC) pw[tid] = powf(P.decay[h], (float)tid);
   float S[MAXD];
-  float* st_base = P.state + (((long long)seq * P.H + h) * D) * Dv;
+  const float* sin_base = Sin + c * u_stride + (long long)h * D * Dv;
 #pragma unroll
-  for (int i = 0; i < MAXD; ++i) S[i] = (colok && i < D) ? st_base[(long long)i * Dv + col] : 0.f;
+  for (int i = 0; i < MAXD; ++i) S[i] = (colok && i < D) ? sin_base[(long long)i * Dv + col] : 0.f;
+  stage_qk<MAXD, true>(P, R, row0, cn, h, Qs, Ks);
+  stage_v(P, row0, cn, h, jb, Vs);
   __syncthreads();
-  const int n = seg_n;
-  const float kscale = 1.f / sqrtf((float)D);
-  const int half = P.rot_dims / 2;
-  for (int c0 = 0; c0 < n; c0 += RC) {
-    const int cn = min(RC, n - c0);
-    // stage the chunk: rows past cn and dims past D are zero, so the loops below run to their full extent
-    for (int idx = tid; idx < RC * MAXD; idx += 256) {
-      const int c = idx / MAXD, d = idx % MAXD;
-      float qv = 0.f, kv = 0.f;
-      if (c < cn && d < D) {
-        const int r = r0 + c0 + c;
-        const float* q = P.proj + (long long)r * P.ld + P.off_q + h * D;
-        const float* k = P.proj + (long long)r * P.ld + P.off_k + h * D;
-        qv = q[d];
-        kv = k[d];
-        if (d < P.rot_dims) {
-          const int i = d < half ? d : d - half;
-          const float ang = (float)R.pos[r] * P.inv_freq[i];
-          const float cs = cosf(ang), sn = sinf(ang);
-          if (d < half) {
-            qv = q[d] * cs - q[d + half] * sn;
-            kv = k[d] * cs - k[d + half] * sn;
-          } else {
-            qv = q[d] * cs + q[i] * sn;
-            kv = k[d] * cs + k[i] * sn;
-          }
-        }
-      }
-      Qs[c][d] = qv;
-      Ks[c][d] = kv * kscale;
-    }
-    for (int idx = tid; idx < RC * 64; idx += 256) {
-      const int c = idx >> 6, jj = idx & 63;
-      const int cc = jb * 64 + jj;
-      Vs[c][jj] = (c < cn && cc < Dv) ? P.proj[(long long)(r0 + c0 + c) * P.ld + P.off_v + h * Dv + cc] : 0.f;
-    }
-    __syncthreads();
 #pragma unroll
-    for (int kx = 0; kx < RC * RC / 256; ++kx) {
-      const int t = (tid >> 5) + 8 * kx, sx = tid & 31;
-      float dot = 0.f;
-      if (sx <= t) {
-#pragma unroll
-        for (int i4 = 0; i4 < MAXD / 4; ++i4) {
-          const f32x4 a = *(const f32x4*)&Qs[t][4 * i4], b = *(const f32x4*)&Ks[sx][4 * i4];
-          dot += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
-        }
-        dot *= pw[t - sx];
-      }
-      As[t][sx] = dot;
-    }
-    __syncthreads();
-    for (int t = g4; t < cn; t += 4) {
-      float inter = 0.f;
+  for (int kx = 0; kx < RC * RC / 256; ++kx) {
+    const int t = (tid >> 5) + 8 * kx, sx = tid & 31;
+    float dot = 0.f;
+    if (sx <= t) {
 #pragma unroll
       for (int i4 = 0; i4 < MAXD / 4; ++i4) {
-        const f32x4 a = *(const f32x4*)&Qs[t][4 * i4];
-        inter += a[0] * S[4 * i4] + a[1] * S[4 * i4 + 1] + a[2] * S[4 * i4 + 2] + a[3] * S[4 * i4 + 3];
+        const f32x4 qa = *(const f32x4*)&Qs[t][4 * i4], kb = *(const f32x4*)&Ks[sx][4 * i4];
+        dot += qa[0] * kb[0] + qa[1] * kb[1] + qa[2] * kb[2] + qa[3] * kb[3];
       }
-      float intra = 0.f;
-#pragma unroll
-      for (int sx = 0; sx < RC; ++sx) intra += As[t][sx] * Vs[sx][j];  // As is zero above the diagonal
-      if (colok) obuf[(long long)(r0 + c0 + t) * ld_o + h * Dv + col] = pw[t + 1] * inter + intra;
+      dot *= pw[t - sx];
     }
-    const float dn = pw[cn];
-#pragma unroll
-    for (int i = 0; i < MAXD; ++i) S[i] *= dn;
-    for (int sx = 0; sx < cn; ++sx) {
-      const float vv = Vs[sx][j] * pw[cn - 1 - sx];
-#pragma unroll
-      for (int i4 = 0; i4 < MAXD / 4; ++i4) {
-        const f32x4 b = *(const f32x4*)&Ks[sx][4 * i4];
-        S[4 * i4] += b[0] * vv;
-        S[4 * i4 + 1] += b[1] * vv;
-        S[4 * i4 + 2] += b[2] * vv;
-        S[4 * i4 + 3] += b[3] * vv;
-      }
-    }
-    __syncthreads();
+    As[t][sx] = dot;
   }
-  if (g4 == 0 && colok) {
+  __syncthreads();
+  for (int t = g4; t < cn; t += 4) {
+    float inter = 0.f;
 #pragma unroll
-    for (int i = 0; i < MAXD; ++i)
-      if (i < D) st_base[(long long)i * Dv + col] = S[i];
+    for (int i4 = 0; i4 < MAXD / 4; ++i4) {
+      const f32x4 qa = *(const f32x4*)&Qs[t][4 * i4];
+      inter += qa[0] * S[4 * i4] + qa[1] * S[4 * i4 + 1] + qa[2] * S[4 * i4 + 2] + qa[3] * S[4 * i4 + 3];
+    }
+    float intra = 0.f;
+#pragma unroll
+    for (int sx = 0; sx < RC; ++sx) intra += As[t][sx] * Vs[sx][j];  // As is zero above the diagonal
+    if (colok) obuf[(long long)(row0 + t) * ld_o + h * Dv + col] = pw[t + 1] * inter + intra;
   }
 }
 // out = o / sqrt(mean_j(o^2) + eps) * silu(gate), one wave per (row, head)
@@ -873,24 +1177,37 @@ __global__ __launch_bounds__(256) void retention_finish_kernel(RetParams P, int 
   for (int jx = lane; jx < P.Dv; jx += 64) st(out + jx, o[jx] * rs * silu(gate[jx]));
 }
 bool retention_chunk_supported(int D, int Dv) { return D > 0 && D <= 128 && Dv > 0 && Dv <= 256; }
-void retention_chunked(const RetParams& P, const StepRows& R, float* obuf, int ld_o, hipStream_t s) {
-  check(R.B > 0 && P.proj && P.state && P.decay && P.out && obuf && ld_o >= P.H * P.Dv && retention_chunk_supported(P.D, P.Dv),
+void retention_chunked(const RetParams& P, const StepRows& R, const RetChunkWs& W, hipStream_t s) {
+  check(R.B > 0 && P.proj && P.state && P.decay && P.out && W.obuf && W.ld_o >= P.H * P.Dv &&
+            retention_chunk_supported(P.D, P.Dv),
         "chunked retention: dim <= 128, vdim <= 256");
   check(P.rot_dims % 2 == 0 && P.rot_dims <= P.D && (P.rot_dims == 0 || P.inv_freq), "retention: bad rotary dims");
+  check(W.chunks && W.nchunks > 0 && W.U && W.Sin && W.u_stride >= (long long)P.H * P.D * P.Dv && W.nchunks <= W.max_chunks,
+        "chunked retention: chunk table or workspace");
   const int NJ = (P.Dv + 63) / 64;
-  dim3 grid(R.B, P.H * NJ);
+  dim3 grid(W.nchunks, P.H * NJ);
   if (P.D <= 64)
-    hipLaunchKernelGGL(retention_chunk_kernel<64>, grid, dim3(256), 0, s, P, R, obuf, ld_o, NJ);
+    hipLaunchKernelGGL(retention_u_kernel<64>, grid, dim3(256), 0, s, P, R, W.chunks, W.U, W.u_stride, NJ);
   else
-    hipLaunchKernelGGL(retention_chunk_kernel<128>, grid, dim3(256), 0, s, P, R, obuf, ld_o, NJ);
-  launched("retention_chunk");
+    hipLaunchKernelGGL(retention_u_kernel<128>, grid, dim3(256), 0, s, P, R, W.chunks, W.U, W.u_stride, NJ);
+  launched("retention_u");
+  const long long elems = (long long)P.H * P.D * P.Dv;
+  hipLaunchKernelGGL(retention_scan_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, s, P, W.chunks, W.nchunks, W.U,
+                     W.Sin, W.u_stride);
+  launched("retention_scan");
+  if (P.D <= 64)
+    hipLaunchKernelGGL(retention_out_kernel<64>, grid, dim3(256), 0, s, P, R, W.chunks, W.Sin, W.u_stride, W.obuf, W.ld_o, NJ);
+  else
+    hipLaunchKernelGGL(retention_out_kernel<128>, grid, dim3(256), 0, s, P, R, W.chunks, W.Sin, W.u_stride, W.obuf, W.ld_o, NJ);
+  launched("retention_out");
   dim3 g2((R.B * P.H + 3) / 4);
   if (P.f32)
-    hipLaunchKernelGGL(retention_finish_kernel<float>, g2, dim3(256), 0, s, P, R.B, obuf, ld_o);
+    hipLaunchKernelGGL(retention_finish_kernel<float>, g2, dim3(256), 0, s, P, R.B, W.obuf, W.ld_o);
   else
-    hipLaunchKernelGGL(retention_finish_kernel<bf16>, g2, dim3(256), 0, s, P, R.B, obuf, ld_o);
+    hipLaunchKernelGGL(retention_finish_kernel<bf16>, g2, dim3(256), 0, s, P, R.B, W.obuf, W.ld_o);
   launched("retention_finish");
 }
+int retention_chunk_rows() { return RC; }
 
 bool retention_supported(int D, int Dv) {
   if (D <= 0 || Dv <= 0 || D > 256 || Dv > 256) return false;

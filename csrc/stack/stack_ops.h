@@ -68,6 +68,19 @@ void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s);
 // softmax(cap(q . k * scale)) v over the first q_len keys of the row's sequence
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s);
 
+// prompt portions on the matrix cores (bfloat16, head sizes 64 / 96 / 128 with dim == vdim): `tiles` is a device
+// table the host builds from the step's rows, per tile {first row, rows <= 32}, rows of one sequence in order
+void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s);
+bool flash_prefill_supported(const AttnParams& P);
+constexpr int FLASH_TILE_ROWS = 32;
+
+// decode steps (M <= 8 rows that fit LDS): C = layer_norm(x) . W^T in one launch; the normed rows also go to hout
+// (matrix dtype). With A (an attention layer): q outputs get the row's query temperature, k and v outputs are
+// also stored at the row's cache slot, so no attn_prepare follows.
+void gemv_ln(const float* x, int E, const float* nw, const float* nb, float eps, const void* W, int M, int N, float* C,
+             int ldc, void* hout, const AttnParams* A, const StepRows* R, int f32, hipStream_t s);
+bool gemv_ln_supported(int M, int E, int f32);
+
 struct RetParams {
   const float* proj;    // [B][ld] float32: q, k, v, g
   int ld, off_q, off_k, off_v, off_g;
@@ -84,9 +97,21 @@ struct RetParams {
 // rows of one sequence are contiguous and in position order; each sequence's state advances through them
 void retention(const RetParams& P, const StepRows& R, hipStream_t s);
 bool retention_supported(int D, int Dv);
-// the same recurrence in chunks (prompt portions): un-normalised o into obuf [B][ld_o] float32, then the unit
-// RMS and the gate in a second launch
-void retention_chunked(const RetParams& P, const StepRows& R, float* obuf, int ld_o, hipStream_t s);
+// the same recurrence in chunks (prompt portions), chunks in parallel around a scan over each sequence's chunk
+// states; `chunks` is a device table the host builds from the step's rows: per chunk {first row, rows (at most
+// retention_chunk_rows()), state slot, flags (1 = first chunk of its sequence's rows, 2 = last)}, a sequence's
+// chunks in row order. The un-normalised o goes through obuf [B][ld_o]; U and Sin hold one state per chunk.
+struct RetChunkWs {
+  const int* chunks;
+  int nchunks, max_chunks;
+  float* U;
+  float* Sin;
+  long long u_stride;   // floats between chunks in U and Sin (>= heads * dim * vdim)
+  float* obuf;
+  int ld_o;
+};
+void retention_chunked(const RetParams& P, const StepRows& R, const RetChunkWs& W, hipStream_t s);
+int retention_chunk_rows();
 bool retention_chunk_supported(int D, int Dv);
 
 struct MoeParams {

@@ -63,14 +63,49 @@ class StackExec:
                              ld_proj=r.proj.shape[1], a=p(r.abuf), ld_a=r.abuf.shape[1], hmid=p(r.hmid),
                              ld_hmid=r.hmid.shape[1], y=p(r.ybuf), eids=p(r.eids), ew=p(r.ew), ld_top=r.eids.shape[1],
                              sgate=p(r.sgate), lrows=p(r.lbuf), obuf=p(r.obuf), ld_obuf=r.obuf.shape[1],
+                             ret_chunks=p(r.d_chunks), ret_max_chunks=r.d_chunks.shape[0], ret_u=p(r.ret_u),
+                             ret_sin=p(r.ret_sin), ret_u_stride=r.ret_u.shape[1],
                              **{"moe_" + k: (v if isinstance(v, int) else p(v)) for k, v in r.moe_ws.items()}))
         e.set_inputs(dict(tokens=p(r.d_tokens), pos=p(r.d_pos), slot=p(r.d_slot), q_len=p(r.d_qlen),
                           q_seq=p(r.d_qseq), block_table=p(r.d_block_table), max_blocks=r.max_blocks,
                           bs=r.block_size, logits=p(r.logits), ld_logits=r.logits.shape[1],
                           logit_idx=p(r.d_logit_idx)))
         self.stages = dict(forward=C.ST_FORWARD, embed=C.ST_EMBED, run=C.ST_RUN, head=C.ST_HEAD)
+        self.chunk_rows = C.retention_chunk_rows()
+        self.tile_rows = C.FLASH_TILE_ROWS
+        e.bind_tiles(p(r.d_tiles), r.d_tiles.shape[0])
+
+    def bind_chunks(self, rows) -> None:
+        """The row tables of the next step: `rows` = (positions, sequence rows) of its B rows as the host
+        uploaded them, or None (the device advanced the rows itself: decode steps). Each sequence's contiguous
+        rows are cut into retention chunks {first row, rows, state slot, first | last flags} and attention query
+        tiles {first row, rows}; without tables the step takes the per-row kernels."""
+        r = self.r
+        self.exe.set_chunks(0)
+        self.exe.set_tiles(0)
+        if rows is None or len(rows[0]) <= 16:
+            return
+        _pos, qseq = rows
+        B, segs, a = len(qseq), [], 0
+        for i in range(1, B + 1):
+            if i == B or qseq[i] != qseq[a]:
+                segs.append((a, i))
+                a = i
+        C, T = self.chunk_rows, self.tile_rows
+        chunks = [(c0, min(C, i - c0), int(qseq[a]), (1 if c0 == a else 0) | (2 if c0 + C >= i else 0))
+                  for a, i in segs for c0 in range(a, i, C)] if r.cfg.has_state else []
+        tiles = [(t0, min(T, i - t0)) for a, i in segs for t0 in range(a, i, T)]
+        if chunks and len(chunks) <= r.d_chunks.shape[0]:
+            r.d_chunks[:len(chunks)].copy_(torch.tensor(chunks, dtype=torch.int32))
+            self.exe.set_chunks(len(chunks))
+        if len(tiles) <= r.d_tiles.shape[0]:
+            r.d_tiles[:len(tiles)].copy_(torch.tensor(tiles, dtype=torch.int32))
+            self.exe.set_tiles(len(tiles))
 
     def run(self, stage: str, layer: int, B: int, n_logits: int = 0, use_idx: bool = False, prefill: bool = False):
+        if stage in ("forward", "embed"):  # a new step: its rows as the host uploaded them, if it did
+            rows, self.r._step_rows = self.r._step_rows, None
+            self.bind_chunks(rows if rows is not None and len(rows[0]) == B else None)
         self.exe.step(self.stages[stage], layer, B, n_logits, use_idx, torch.cuda.current_stream().cuda_stream)
 
 
@@ -119,7 +154,7 @@ class StackRunner(Runner):
         self.x0 = torch.zeros(max_batch, E, **f32)          # the embedding output (re-enters at every pass)
         self.hbuf = torch.zeros(max_batch, E, **tt)         # normed activations, the input projection's operand
         self.catbuf = torch.zeros(max_batch, 2 * E, **tt)   # [x; x0], the pass-opening projection's operand
-        self.proj = torch.zeros(max_batch, max(L["n_in"] for L in self.w.layers), **f32)
+        self.proj = torch.zeros(max_batch, (max(L["n_in"] for L in self.w.layers) + 3) // 4 * 4, **f32)  # rows 16-byte aligned
         self.abuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **tt)
         self.hmid = torch.zeros(max_batch, max([f.top * f.ff + f.shared_ff for f in mlps], default=1), **tt)
         self.ybuf = torch.zeros(max_batch, E, **f32)
@@ -128,6 +163,14 @@ class StackRunner(Runner):
         self.sgate = torch.zeros(max_batch, **f32)
         self.lbuf = torch.zeros(max_batch, E, **tt)
         self.obuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **f32)  # retention, before its norm
+        # chunked retention of prompt portions: the chunk table and one state per chunk (its U, its incoming state)
+        rets = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_RETENTION]
+        n_ch = max_batch // 32 + max_seqs + 1 if rets and max_batch > 16 else 1
+        self.d_chunks = torch.zeros(n_ch, 4, **i32)
+        self.d_tiles = torch.zeros(max_batch // 32 + max_seqs + 1, 2, **i32)  # attention query tiles of a step
+        self.ret_u = torch.zeros(n_ch, max([m.heads * m.dim * m.vdim for m in rets], default=1) if n_ch > 1 else 1, **f32)
+        self.ret_sin = torch.zeros_like(self.ret_u)
+        self._step_rows = None  # (positions, sequence rows) of the rows last uploaded, until a step consumes them
         # routed feed-forward of prompt portions (bfloat16): pairs sorted by expert, per-expert matrix-core products
         self.moe_ws = {}
         if mlps and T == torch.bfloat16:
@@ -168,6 +211,11 @@ class StackRunner(Runner):
         if self._closed:
             raise RuntimeError("runner is closed")
         self.exe.run("forward", 0, B, n_logits, use_idx, prefill)
+
+    def _upload(self, arr, tokens):
+        super()._upload(arr, tokens)
+        if arr.shape[1]:
+            self._step_rows = (arr[0].tolist(), arr[3].tolist())
 
     def split_plan(self, B: int) -> tuple[int, int]:
         return 1, 0

@@ -241,6 +241,29 @@ def test_other_sizes(tmp_path, device):
         bc.check(bc.run_cuts(r, toks, [140] + list(range(141, 151))), want, dtype, "decode")
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dim", [64, 96, 128])
+def test_matrix_core_head_sizes(tmp_path, device, dim):
+    """Head sizes that the matrix-core kernels take on a GPU (bfloat16 prompt portions: query tiles of 32 rows,
+    keys by 32), grouped and ungrouped heads, a retention layer between: whole prompt, portions that end inside
+    a tile, single tokens, and two sequences in one step."""
+    layers = [(bc.attn(heads=4, kv_heads=2, dim=dim, vdim=dim, scale=dim ** -0.5, softcap=25.0, coef=0.3, every=32), bc.moe(ff=32, shared_ff=32)),
+              (bc.ret(heads=2, dim=64, vdim=128, decay=(0.97, 0.999), rot_dims=64, base=1e4), None),
+              (bc.attn(heads=2, kv_heads=2, dim=dim, vdim=dim, scale=2.0 * dim ** -0.5, softcap=0.0, coef=0.0), None)]
+    m = bc.Model(tmp_path, bc.config(layers, width=128, vocab=120, mult=0.5), seed=dim)
+    a, b = bc.tokens(170, 120, seed=1), bc.tokens(75, 120, seed=2)
+    wa, wb = m.oracle(a)[0], m.oracle(b)[0]
+    for dtype in BOTH:
+        r = m.runner(device, dtype, max_batch=256, kv_tokens=512)
+        bc.check(bc.run_cuts(r, a, [170]), wa, dtype, "whole")
+        bc.check(bc.run_cuts(r, a, [33, 100, 131, 132, 170]), wa, dtype, "portions")
+        sa, sb = r.new_sequence(), r.new_sequence()
+        o1 = r.step_entries([(sa, a[:90], list(range(90))), (sb, b[:40], list(range(40)))]).float().cpu().numpy()
+        o2 = r.step_entries([(sa, a[90:], list(range(80))), (sb, b[40:], list(range(35)))]).float().cpu().numpy()
+        bc.check(np.concatenate([o1[:90], o2[:80]]), wa, dtype, "first of two sequences")
+        bc.check(np.concatenate([o1[90:], o2[80:]]), wb, dtype, "second of two sequences")
+
+
 # ------------------------------------------------------------------ generation through the engine's entry points
 def greedy_oracle(m, prompt, n):
     toks = list(prompt)
