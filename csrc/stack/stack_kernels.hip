@@ -8,6 +8,7 @@
 #include <stdexcept>
 #include <string>
 
+#include "../kernels/wave_shuffle.h"
 #include "stack_ops.h"
 
 namespace omx {
@@ -34,14 +35,23 @@ __device__ __forceinline__ float ld(const bf16* p) { return bf2f(p->v); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16* p, float v) { p->v = f2bf(v); }
 
+// butterfly reductions on DPP / permlane exchanges (wave_shuffle.h): no LDS round trip per dependent step
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  v += xor_shfl<32>(v);
+  v += xor_shfl<16>(v);
+  v += xor_shfl<8>(v);
+  v += xor_shfl<4>(v);
+  v += xor_shfl<2>(v);
+  v += xor_shfl<1>(v);
   return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  v = fmaxf(v, xor_shfl<32>(v));
+  v = fmaxf(v, xor_shfl<16>(v));
+  v = fmaxf(v, xor_shfl<8>(v));
+  v = fmaxf(v, xor_shfl<4>(v));
+  v = fmaxf(v, xor_shfl<2>(v));
+  v = fmaxf(v, xor_shfl<1>(v));
   return v;
 }
 // sum over a block of 256 threads; every thread gets the result. red: 4 floats of LDS
@@ -598,8 +608,17 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
     float dot[RQ];
 #pragma unroll
     for (int r = 0; r < RQ; ++r) dot[r] = 0.f;
+    if (valid) rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
+    // the first UB keys' value rows are requested ahead of the K rows: one round trip brings both
+    constexpr int UB = 64 / DC;
+    float v0[UB][DC];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const T* vr = vc + (long long)__builtin_amdgcn_readlane(rowidx, u) * P.Dv;  // a key past the end: row 0, weight 0
+#pragma unroll
+      for (int c = 0; c < DC; ++c) v0[u][c] = (lane + 64 * c < P.Dv) ? ld(vr + lane + 64 * c) : 0.f;
+    }
     if (valid) {
-      rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
       const T* kr = kc + (long long)rowidx * P.D;
       if (vec) {
         for (int d0 = 0; d0 < P.D; d0 += 64) {  // 64 dims of the row in flight at a time
@@ -643,15 +662,20 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
       for (int c = 0; c < DC; ++c) acc[r][c] *= corr;
       m[r] = mn;
     }
-    // values: UB keys' rows in flight at a time (a key past the group's end reads row 0 with weight 0)
-    constexpr int UB = 32 / DC;
     const int cnt = min(64, n - t0);
-    for (int j0 = 0; j0 < cnt; j0 += UB) {
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+#pragma unroll
+      for (int r = 0; r < RQ; ++r) {
+        const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p[r]), u));  // 0 for keys past the end
+#pragma unroll
+        for (int c = 0; c < DC; ++c) acc[r][c] += pj * v0[u][c];
+      }
+    for (int j0 = UB; j0 < cnt; j0 += UB) {  // wide values: the rest of the group, UB rows in flight at a time
       float v[UB][DC];
 #pragma unroll
       for (int u = 0; u < UB; ++u) {
-        const int rj = __shfl(rowidx, j0 + u, 64);
-        const T* vr = vc + (long long)rj * P.Dv;
+        const T* vr = vc + (long long)__builtin_amdgcn_readlane(rowidx, j0 + u) * P.Dv;
 #pragma unroll
         for (int c = 0; c < DC; ++c) v[u][c] = (lane + 64 * c < P.Dv) ? ld(vr + lane + 64 * c) : 0.f;
       }
@@ -659,7 +683,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
       for (int u = 0; u < UB; ++u)
 #pragma unroll
         for (int r = 0; r < RQ; ++r) {
-          const float pj = __shfl(p[r], j0 + u, 64);  // 0 for keys past the end
+          const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p[r]), j0 + u));
 #pragma unroll
           for (int c = 0; c < DC; ++c) acc[r][c] += pj * v[u][c];
         }
@@ -842,7 +866,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
       pr[r] = vis ? sc : -1e30f;
       mx = fmaxf(mx, pr[r]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = fmaxf(mx, xor_shfl<32>(mx));
     const float mn = fmaxf(mi, mx);
     const float corr = fast_exp(fmaxf(mi - mn, -100.f));
     float sum = 0.f;
@@ -851,7 +875,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
       pr[r] = pr[r] > -1e29f ? fast_exp(pr[r] - mn) : 0.f;
       sum += pr[r];
     }
-    sum += __shfl_xor(sum, 32, 64);
+    sum += xor_shfl<32>(sum);
     li = li * corr + sum;
     mi = mn;
 #pragma unroll

@@ -243,6 +243,31 @@ def cmd_run(a):
             msgs.append({"role": "assistant", "content": "".join(out)})
 
 
+def cmd_tokens(a):
+    """Generate token ids from token ids with a model file or folder, straight through the engine (no server, no
+    tokenizer): `ollama tokens MODEL --ids "5 17 3" --num-predict 16`. The runner class follows the model
+    (engine.load_runner): a GGUF file, or a folder with config.json + model.safetensors."""
+    from .engine import load_runner
+    from .engine.sampling import SamplingOptions
+    ids = [int(x) for x in a.ids.replace(",", " ").split()]
+    if not ids:
+        raise SystemExit("tokens: --ids needs at least one token id")
+    kw = dict(max_batch=a.chunk, max_seqs=2, ctx=len(ids) + a.num_predict + 16)
+    if a.device:
+        kw["device"] = a.device
+    if a.dtype:
+        kw["dtype"] = a.dtype
+    r = load_runner(a.model, **kw)
+    bad = [t for t in ids if not 0 <= t < r.cfg.n_vocab]
+    if bad:
+        raise SystemExit(f"tokens: ids outside the vocabulary (0..{r.cfg.n_vocab - 1}): {bad[:5]}")
+    r.warmup()
+    o = SamplingOptions(temperature=a.temperature, seed=a.seed, repeat_penalty=a.repeat_penalty)
+    out = list(r.generate(r.new_sequence(), ids, o, max_tokens=a.num_predict))
+    print(" ".join(str(t) for t in out))
+    r.close()
+
+
 def _stats(ev):
     ec, ed = ev.get("eval_count", 0), ev.get("eval_duration", 1)
     pc, pd = ev.get("prompt_eval_count", 0), ev.get("prompt_eval_duration", 1)
@@ -287,6 +312,17 @@ def main(argv=None):
     s.add_argument("model")
     s.add_argument("-f", "--file", default="Modelfile")
     s.set_defaults(f=cmd_create)
+    s = sub.add_parser("tokens", help="generate token ids from token ids through the engine (GGUF file or model folder)")
+    s.add_argument("model")
+    s.add_argument("--ids", required=True, help="prompt token ids, separated by spaces or commas")
+    s.add_argument("--num-predict", type=int, default=16)
+    s.add_argument("--temperature", type=float, default=0.0)
+    s.add_argument("--repeat-penalty", type=float, default=1.0)
+    s.add_argument("--seed", type=int, default=0)
+    s.add_argument("--chunk", type=int, default=512, help="rows per prefill forward")
+    s.add_argument("--device", default="", help="cuda | cpu (default: the GPU when there is one)")
+    s.add_argument("--dtype", default="", help="layer-list models: bfloat16 (default) | float32")
+    s.set_defaults(f=cmd_tokens)
     s = sub.add_parser("stop")
     s.add_argument("model")
     s.set_defaults(f=cmd_stop)

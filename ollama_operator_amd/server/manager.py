@@ -152,7 +152,7 @@ class ModelManager:
             return lm
 
     def _load(self, name: ModelName, m, num_ctx: int) -> LoadedModel:
-        from ..engine.runner import Runner
+        from ..engine import load_runner
         from ..models.clip import ImageIds
         from ..gguf import read_gguf
         t0 = time.perf_counter()
@@ -187,7 +187,7 @@ class ModelManager:
             runner = load_tp_runner(self.tp_world, path, max_batch=chunk, max_seqs=max_seqs, ctx=ctx,
                                     ext_rows=ext_rows)
         else:
-            runner = Runner(path, device=self.device, max_batch=chunk, max_seqs=max_seqs, ctx=ctx, ext_rows=ext_rows)
+            runner = load_runner(path, device=self.device, max_batch=chunk, max_seqs=max_seqs, ctx=ctx, ext_rows=ext_rows)
         if vision is not None and vision.out_dim != runner.cfg.n_embd:
             raise StoreError(f"projector output width {vision.out_dim} != model embedding width {runner.cfg.n_embd}")
         runner.warmup()

@@ -309,6 +309,46 @@ def test_scheduler_batches_requests(std, device):
         sch.close()
 
 
+def test_command_line_generates_token_ids(std, capsys):
+    """`ollama tokens MODEL --ids ...`: the command line picks the runner class by the model and generates
+    through `Runner.generate`."""
+    from ollama_operator_amd import cli
+    prompt = bc.tokens(9, 96, seed=90)
+    cli.main(["tokens", std.path, "--ids", " ".join(map(str, prompt)), "--num-predict", "5", "--device", "cpu",
+              "--dtype", "float32"])
+    out = capsys.readouterr().out.strip().splitlines()[-1]
+    assert [int(t) for t in out.split()] == greedy_oracle(std, prompt, 5)
+
+
+def test_trace_replay_program(std, tmp_path):
+    """bin/trace_run on the CPU twin: steps on standard input, logits files and `done` lines out; a request
+    that sits out a step, one that ends and gives its slot back."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b = bc.tokens(30, 96, seed=91), bc.tokens(12, 96, seed=92)
+    steps = [dict(step=0, entries=[dict(id="a", tokens=a[:20], want=[0, 19])], end=[]),
+             dict(step=1, entries=[dict(id="b", tokens=b, want=[11])], end=["b"]),
+             dict(step=2, entries=[dict(id="a", tokens=a[20:], want=[9])], end=["a"]),
+             dict(step=3, entries=[dict(id="c", tokens=b[:2], want=[])], end=["c"])]
+    out = tmp_path / "out"
+    p = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", std.path, "--dtype", "float32", "--out", str(out),
+                        "--max-tokens", "64", "--device", "cpu"], input="".join(json.dumps(x) + "\n" for x in steps),
+                       capture_output=True, text=True, timeout=300, env={**os.environ, "PYTHON": sys.executable})
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+    wa, wb = std.oracle(a)[0], std.oracle(b)[0]
+    got0 = np.fromfile(out / "0.f32", "<f4").reshape(2, 96)
+    got1 = np.fromfile(out / "1.f32", "<f4").reshape(1, 96)
+    got2 = np.fromfile(out / "2.f32", "<f4").reshape(1, 96)
+    bc.check(got0, wa[[0, 19]], "float32", "step 0")
+    bc.check(got1, wb[[11]], "float32", "step 1")
+    bc.check(got2, wa[[29]], "float32", "step 2")
+    assert not (out / "3.f32").exists()
+
+
 # ------------------------------------------------------------------ kernels on their own (GPU)
 @pytest.mark.gpu
 def test_gemm_kernels_against_torch():
