@@ -229,7 +229,8 @@ def test_first_tokens(std, device):
 def test_other_sizes(tmp_path, device):
     """Sizes off the beaten track: a width and head sizes that are not multiples of 8 (no vector loads), one
     query head per key/value head, more rows than one tile, a wide vocabulary, no caps, residual factor 1."""
-    layers = [(bc.attn(heads=3, kv_heads=3, dim=10, vdim=6, scale=0.3, softcap=0.0, coef=0.0), bc.moe(experts=3, top=2, ff=10, shared_ff=6)),
+    layers = [(bc.attn(heads=3, kv_heads=3, dim=10, vdim=6, scale=0.3, softcap=0.0, coef=0.0),
+               bc.moe(experts=3, top=2, ff=10, shared_ff=6)),
               (bc.ret(heads=2, dim=10, vdim=14, decay=(0.8, 0.95), rot_dims=4), None),
               (bc.attn(heads=8, kv_heads=2, dim=64, vdim=64, every=1), bc.moe(experts=9, top=4, ff=64, shared_ff=128))]
     m = bc.Model(tmp_path, bc.config(layers, width=52, vocab=203, mult=1.0, cap=0.0, eps=1e-3), seed=13)
@@ -247,7 +248,8 @@ def test_matrix_core_head_sizes(tmp_path, device, dim):
     """Head sizes that the matrix-core kernels take on a GPU (bfloat16 prompt portions: query tiles of 32 rows,
     keys by 32), grouped and ungrouped heads, a retention layer between: whole prompt, portions that end inside
     a tile, single tokens, and two sequences in one step."""
-    layers = [(bc.attn(heads=4, kv_heads=2, dim=dim, vdim=dim, scale=dim ** -0.5, softcap=25.0, coef=0.3, every=32), bc.moe(ff=32, shared_ff=32)),
+    layers = [(bc.attn(heads=4, kv_heads=2, dim=dim, vdim=dim, scale=dim ** -0.5, softcap=25.0, coef=0.3, every=32),
+               bc.moe(ff=32, shared_ff=32)),
               (bc.ret(heads=2, dim=64, vdim=128, decay=(0.97, 0.999), rot_dims=64, base=1e4), None),
               (bc.attn(heads=2, kv_heads=2, dim=dim, vdim=dim, scale=2.0 * dim ** -0.5, softcap=0.0, coef=0.0), None)]
     m = bc.Model(tmp_path, bc.config(layers, width=128, vocab=120, mult=0.5), seed=dim)
