@@ -27,7 +27,7 @@ void StackExecutor::validate() const {
       need(L.dim <= 256 && L.vdim <= 256 && L.kv_heads > 0 && L.heads % L.kv_heads == 0, "attention head sizes");
     } else {
       need(r.state && L.decay, "retention run without a state");
-      need(retention_supported(L.dim, L.vdim), "retention head sizes (dim, vdim <= 256, dim * vdim <= 16384)");
+      need(retention_supported(L.dim, L.vdim) || retention_general_supported(L.dim, L.vdim), "retention head sizes (<= 1024)");
       need(L.rot_dims == 0 || L.inv_freq, "retention rotary table missing");
     }
     if (L.experts) {

@@ -168,6 +168,7 @@ struct QkvEpi {
   void* vc;
 };
 constexpr int LN_LDS_BYTES = 32768;
+constexpr int LN_RW = 4;  // weight rows per wave
 template <typename T>
 __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ x, int E, const float* __restrict__ nw,
                                                       const float* __restrict__ nb, float eps, const T* __restrict__ W,
@@ -194,12 +195,53 @@ __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ 
     }
   }
   __syncthreads();
-  const int n = blockIdx.x * 4 + (tid >> 6);
-  if (n >= N) return;
-  const T* w = W + (long long)n * E;
+  // LN_RW weight rows per wave, streamed together (independent loads in flight), against every activation row
+  const int n0 = (blockIdx.x * 4 + (tid >> 6)) * LN_RW;
+  if (n0 >= N) return;
   for (int m = 0; m < M; ++m) {
-    float acc = wave_dot<T>(w, hs + (long long)m * E, E, lane, vec != 0);
-    if (lane == 0) {
+    float accs[LN_RW];
+#pragma unroll
+    for (int u = 0; u < LN_RW; ++u) accs[u] = 0.f;
+    const T* xr = hs + (long long)m * E;
+    if (vec) {
+      constexpr int PER = 16 / (int)sizeof(T);
+      for (int k = lane * PER; k < E; k += 64 * PER) {
+        float xv[8], wv[LN_RW][8];
+#pragma unroll
+        for (int u = 0; u < LN_RW; ++u) {
+          const T* w = W + (long long)min(n0 + u, N - 1) * E + k;
+          if constexpr (PER == 8) {
+            load8<T>(w, wv[u]);
+          } else {
+            const f32x4 t4 = *(const f32x4*)w;
+            wv[u][0] = t4[0], wv[u][1] = t4[1], wv[u][2] = t4[2], wv[u][3] = t4[3];
+          }
+        }
+        if constexpr (PER == 8) {
+          load8<T>(xr + k, xv);
+        } else {
+          const f32x4 t4 = *(const f32x4*)(xr + k);
+          xv[0] = t4[0], xv[1] = t4[1], xv[2] = t4[2], xv[3] = t4[3];
+        }
+#pragma unroll
+        for (int u = 0; u < LN_RW; ++u)
+#pragma unroll
+          for (int i = 0; i < PER; ++i) accs[u] += wv[u][i] * xv[i];
+      }
+    } else {
+      for (int k = lane; k < E; k += 64) {
+        const float xv = ld(xr + k);
+#pragma unroll
+        for (int u = 0; u < LN_RW; ++u) accs[u] += ld(W + (long long)min(n0 + u, N - 1) * E + k) * xv;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < LN_RW; ++u) accs[u] = wave_sum(accs[u]);
+#pragma unroll
+    for (int u = 0; u < LN_RW; ++u) {
+    const int n = n0 + u;
+    float acc = accs[u];
+    if (lane == 0 && n < N) {
       if (q.on) {
         if (n >= q.off_q && n < q.off_q + q.n_q) {
           if (q.coef != 0.f) acc *= 1.f + q.coef * logf(floorf((float)(q.pos[m] + 1) / (float)q.every) + 1.f);
@@ -215,6 +257,7 @@ __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ 
       }
       C[(long long)m * ldc + n] = acc;
     }
+    }
   }
 }
 bool gemv_ln_supported(int M, int E, int f32) { return M > 0 && M <= 8 && (long long)M * E * (f32 ? 4 : 2) <= LN_LDS_BYTES; }
@@ -227,7 +270,7 @@ void gemv_ln(const float* x, int E, const float* nw, const float* nb, float eps,
     q = QkvEpi{1, A->off_q, A->H * A->D, A->off_k, A->G * A->D, A->off_v, A->G * A->Dv, A->G, A->D, A->Dv, R->bs,
                A->qtemp_coef, A->qtemp_every, R->pos, R->slot, A->kc, A->vc};
   }
-  dim3 grid((N + 3) / 4);
+  dim3 grid((N + 4 * LN_RW - 1) / (4 * LN_RW));
   if (f32)
     hipLaunchKernelGGL(gemv_ln_kernel<float>, grid, dim3(256), 0, s, x, E, nw, nb, eps, (const float*)W, M, N, C, ldc,
                        (float*)hout, q, (int)(E % 4 == 0 && ((uintptr_t)W & 15) == 0));
@@ -730,6 +773,157 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
     }
   }
 }
+// ---- decode steps: one block per (row, query head); its four waves take the 64-key groups in turn and merge
+// through LDS. Within a group lane j scores key j (its own K row against the query in LDS); for the values the
+// lanes regroup as (key quarter kq, dim group dq): lane (kq, dq) walks 16 keys for DPL consecutive value dims
+// (weights and row indices come from LDS), so a group costs 16 short iterations instead of 64, and the four
+// quarters meet in two lane exchanges. The serial instruction count per wave is what bounds a decode step.
+template <typename T, int DPL>
+__global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, StepRows R, int vec, int vvec) {
+  __shared__ __attribute__((aligned(16))) float qs[ATT_MAXD];
+  __shared__ float ps[4][64];
+  __shared__ int rs[4][64];
+  __shared__ float mg[4][2];
+  __shared__ float ag[4][16 * DPL];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int b = blockIdx.x / P.H, h = blockIdx.x % P.H;
+  const int g = h / (P.H / P.G);
+  for (int d = threadIdx.x; d < P.D; d += 256) qs[d] = P.proj[(long long)b * P.ld + P.off_q + h * P.D + d];
+  const int n = R.q_len[b];
+  const int* bt = R.block_table + (long long)R.q_seq[b] * R.max_blocks;
+  const T* kc = (const T*)P.kc;
+  const T* vc = (const T*)P.vc;
+  const int kq = lane >> 4, dq = lane & 15;
+  float m = -INFINITY, l = 0.f, acc[DPL];
+#pragma unroll
+  for (int c = 0; c < DPL; ++c) acc[c] = 0.f;
+  __syncthreads();
+  for (int t0 = 64 * wv; t0 < n; t0 += 256) {
+    const int t = t0 + lane;
+    const bool valid = t < n;
+    int rowidx = 0;
+    float dot = 0.f;
+    if (valid) {
+      rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
+      const T* kr = kc + (long long)rowidx * P.D;
+      if (vec) {
+        for (int d0 = 0; d0 < P.D; d0 += 64) {
+          float k8[8][8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) load8<T>(kr + min(d0 + 8 * u, P.D - 8), k8[u]);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int d = d0 + 8 * u;
+            if (d < P.D) {
+              const f32x4 qa = *(const f32x4*)&qs[d], qb = *(const f32x4*)&qs[d + 4];
+              dot += qa[0] * k8[u][0] + qa[1] * k8[u][1] + qa[2] * k8[u][2] + qa[3] * k8[u][3] + qb[0] * k8[u][4] +
+                     qb[1] * k8[u][5] + qb[2] * k8[u][6] + qb[3] * k8[u][7];
+            }
+          }
+        }
+      } else {
+        for (int d = 0; d < P.D; ++d) dot += qs[d] * ld(kr + d);
+      }
+    }
+    float sc = -INFINITY;
+    if (valid) {
+      sc = dot * P.scale;
+      if (P.softcap != 0.f) sc = P.softcap * tanhf(sc / P.softcap);
+    }
+    const float mn = fmaxf(m, wave_max(sc));
+    const float corr = expf(m - mn);
+    const float p = valid ? expf(sc - mn) : 0.f;
+    l = l * corr + wave_sum(p);
+    m = mn;
+    ps[wv][lane] = p;
+    rs[wv][lane] = rowidx;  // a key past the end: row 0 with weight 0
+#pragma unroll
+    for (int c = 0; c < DPL; ++c) acc[c] *= corr;
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
+    float v[16][DPL];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const T* vr = vc + (long long)rs[wv][kq * 16 + i] * P.Dv + dq * DPL;
+      if (vvec) {
+        if (dq * DPL < P.Dv) {
+          if constexpr (DPL == 4 && sizeof(T) == 2) {
+            const unsigned long long w = *(const unsigned long long*)vr;
+            v[i][0] = __uint_as_float((unsigned)(w << 16));
+            v[i][1] = __uint_as_float((unsigned)w & 0xffff0000u);
+            v[i][2] = __uint_as_float((unsigned)(w >> 16) & 0xffff0000u);
+            v[i][3] = __uint_as_float((unsigned)(w >> 32) & 0xffff0000u);
+          } else {
+#pragma unroll
+            for (int c8 = 0; c8 < DPL; c8 += 8) load8<T>(vr + c8, &v[i][c8]);
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < DPL; ++c) v[i][c] = 0.f;
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < DPL; ++c) v[i][c] = (dq * DPL + c < P.Dv) ? ld(vr + c) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float pj = ps[wv][kq * 16 + i];
+#pragma unroll
+      for (int c = 0; c < DPL; ++c) acc[c] += pj * v[i][c];
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  // the four key quarters of the wave, then the four waves of the block
+#pragma unroll
+  for (int c = 0; c < DPL; ++c) {
+    acc[c] += xor_shfl<16>(acc[c]);
+    acc[c] += xor_shfl<32>(acc[c]);
+  }
+  if (lane == 0) {
+    mg[wv][0] = m;
+    mg[wv][1] = l;
+  }
+  if (kq == 0) {
+#pragma unroll
+    for (int c = 0; c < DPL; ++c) ag[wv][dq * DPL + c] = acc[c];
+  }
+  __syncthreads();
+  if (wv != 0 || kq != 0) return;
+  float M = -INFINITY;
+  for (int w = 0; w < 4; ++w) M = fmaxf(M, mg[w][0]);
+  float L = 0.f;
+#pragma unroll
+  for (int c = 0; c < DPL; ++c) acc[c] = 0.f;
+  for (int w = 0; w < 4; ++w) {
+    const float f = expf(mg[w][0] - M);  // a wave without keys: exp(-inf) = 0
+    L += mg[w][1] * f;
+#pragma unroll
+    for (int c = 0; c < DPL; ++c) acc[c] += ag[w][dq * DPL + c] * f;
+  }
+  T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
+  const float inv = 1.f / L;
+#pragma unroll
+  for (int c = 0; c < DPL; ++c)
+    if (dq * DPL + c < P.Dv) st(out + dq * DPL + c, acc[c] * inv);
+}
+template <typename T>
+static void launch_attention_decode(const AttnParams& P, const StepRows& R, hipStream_t s) {
+  const int vec = P.D % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
+  dim3 grid(R.B * P.H);
+  const int per = 16 / (int)sizeof(T);  // elements of a 16-byte load
+  if (P.Dv <= 64) {
+    const int vvec = P.Dv % 4 == 0 && (sizeof(T) == 2 ? 1 : 0) && ((uintptr_t)P.vc & 15) == 0;  // 8-byte pieces (bf16)
+    hipLaunchKernelGGL((attention_decode_kernel<T, 4>), grid, dim3(256), 0, s, P, R, vec, sizeof(T) == 2 ? vvec : 0);
+  } else if (P.Dv <= 128) {
+    const int vvec = P.Dv % 8 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
+    hipLaunchKernelGGL((attention_decode_kernel<T, 8>), grid, dim3(256), 0, s, P, R, vec, vvec);
+  } else {
+    const int vvec = P.Dv % 16 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
+    hipLaunchKernelGGL((attention_decode_kernel<T, 16>), grid, dim3(256), 0, s, P, R, vec, vvec);
+  }
+}
+
 template <typename T, int RQ, int DC>
 static void launch_attention_rd(const AttnParams& P, const StepRows& R, int nbatch, int vec, hipStream_t s) {
   const int items = R.B * P.G * nbatch;
@@ -938,10 +1132,16 @@ void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && P.out,
         "attention: head sizes up to 256, heads a multiple of key/value heads");
-  if (P.f32)
+  if (R.B * P.H <= 1024) {  // decode steps (and short portions): a block per (row, head)
+    if (P.f32)
+      launch_attention_decode<float>(P, R, s);
+    else
+      launch_attention_decode<bf16>(P, R, s);
+  } else if (P.f32) {
     launch_attention<float>(P, R, s);
-  else
+  } else {
     launch_attention<bf16>(P, R, s);
+  }
   launched("attention");
 }
 
@@ -1233,6 +1433,57 @@ void retention_chunked(const RetParams& P, const StepRows& R, const RetChunkWs& 
 }
 int retention_chunk_rows() { return RC; }
 
+// Any head size up to RG_MAX: the state stays in global memory, thread j walks column j of it (reads and writes
+// of a row of S are contiguous across threads). Slow, and only taken when the register kernels do not fit.
+constexpr int RG_MAX = 1024;
+template <typename T>
+__global__ __launch_bounds__(256) void retention_general_kernel(RetParams P, StepRows R) {
+  __shared__ float qs[RG_MAX], ks[RG_MAX], os[RG_MAX], red[4];
+  const int r0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int seq = R.q_seq[r0];
+  if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;
+  const int D = P.D, Dv = P.Dv, half = P.rot_dims / 2;
+  float* S = P.state + (((long long)seq * P.H + h) * D) * Dv;
+  const float dec = P.decay[h], kscale = 1.f / sqrtf((float)D);
+  for (int r = r0; r < R.B && R.q_seq[r] == seq; ++r) {
+    const float* row = P.proj + (long long)r * P.ld;
+    for (int d = tid; d < D; d += 256) {
+      const float* q = row + P.off_q + h * D;
+      const float* k = row + P.off_k + h * D;
+      float qv = q[d], kv = k[d];
+      if (d < P.rot_dims) {
+        const int i = d < half ? d : d - half;
+        const float ang = (float)R.pos[r] * P.inv_freq[i];
+        const float c = cosf(ang), sn = sinf(ang);
+        const float sg = d < half ? -1.f : 1.f;
+        const int pd = d < half ? d + half : d - half;
+        qv = q[d] * c + sg * q[pd] * sn;
+        kv = k[d] * c + sg * k[pd] * sn;
+      }
+      qs[d] = qv;
+      ks[d] = kv * kscale;
+    }
+    __syncthreads();
+    float sq = 0.f;
+    for (int j = tid; j < Dv; j += 256) {
+      const float vj = row[P.off_v + h * Dv + j];
+      float o = 0.f;
+      for (int i = 0; i < D; ++i) {
+        const float sv = dec * S[(long long)i * Dv + j] + ks[i] * vj;
+        S[(long long)i * Dv + j] = sv;
+        o += sv * qs[i];
+      }
+      os[j] = o;
+      sq += o * o;
+    }
+    const float ms = block_sum256(sq, red) / (float)Dv;
+    for (int j = tid; j < Dv; j += 256)
+      st((T*)P.out + (long long)r * P.ld_out + h * Dv + j, os[j] / sqrtf(ms + P.eps) * silu(row[P.off_g + h * Dv + j]));
+    __syncthreads();
+  }
+}
+bool retention_general_supported(int D, int Dv) { return D > 0 && Dv > 0 && D <= RG_MAX && Dv <= RG_MAX; }
+
 bool retention_supported(int D, int Dv) {
   if (D <= 0 || Dv <= 0 || D > 256 || Dv > 256) return false;
   const int ng = 256 / Dv;
@@ -1252,9 +1503,18 @@ static void launch_retention(const RetParams& P, const StepRows& R, hipStream_t 
     hipLaunchKernelGGL((retention_kernel<T, 64>), grid, dim3(256), 0, s, P, R);
 }
 void retention(const RetParams& P, const StepRows& R, hipStream_t s) {
-  check(R.B > 0 && P.proj && P.state && P.decay && P.out && retention_supported(P.D, P.Dv),
-        "retention: head sizes up to 256 with dim * vdim <= 16384");
+  check(R.B > 0 && P.proj && P.state && P.decay && P.out && (retention_supported(P.D, P.Dv) ||
+        retention_general_supported(P.D, P.Dv)), "retention: head sizes up to 1024");
   check(P.rot_dims % 2 == 0 && P.rot_dims <= P.D && (P.rot_dims == 0 || P.inv_freq), "retention: bad rotary dims");
+  if (!retention_supported(P.D, P.Dv)) {
+    dim3 grid(R.B, P.H);
+    if (P.f32)
+      hipLaunchKernelGGL(retention_general_kernel<float>, grid, dim3(256), 0, s, P, R);
+    else
+      hipLaunchKernelGGL(retention_general_kernel<bf16>, grid, dim3(256), 0, s, P, R);
+    launched("retention_general");
+    return;
+  }
   if (P.f32)
     launch_retention<float>(P, R, s);
   else
@@ -1496,19 +1756,40 @@ __global__ __launch_bounds__(256) void moe_route_experts_kernel(MoeParams P, int
     if (f < P.Fs && lane == 0) st(hm + P.top * P.F + f, silu(row[P.off_sgate + f]) * row[P.off_sup + f]);
     return;
   }
-  if (threadIdx.x == 0) {
-    route_row(P, row, ids, val);
-    if (blockIdx.x == 0 && jj == 0) {
-      for (int q = 0; q < P.top; ++q) {
-        P.eids[(long long)b * P.ld_top + q] = ids[q];
-        P.ew[(long long)b * P.ld_top + q] = val[q];
-      }
-      if (P.Fs > 0) P.sgate[b] = sigmoidf(row[P.off_sg]);
+  int e;
+  if (P.X <= 64) {
+    // every wave routes the row itself, one expert per lane: `top` rounds of (maximum, lowest lane that holds it)
+    float z = lane < P.X ? row[P.off_router + lane] + P.router_b[lane] : -INFINITY;
+    float mx0 = 0.f, sum = 0.f, mine = 0.f;
+    e = 0;
+    for (int q = 0; q < P.top; ++q) {
+      const float mx = wave_max(z);
+      const int who = __ffsll((unsigned long long)__ballot(z == mx)) - 1;
+      if (q == 0) mx0 = mx;
+      const float w = expf(mx - mx0);
+      sum += w;
+      if (q == jj) e = who;
+      if (lane == q) mine = w;       // lane q keeps the q-th weight (top <= 16 < 64)
+      if (threadIdx.x == 0 && blockIdx.x == 0 && jj == 0) P.eids[(long long)b * P.ld_top + q] = who;
+      if (lane == who) z = -INFINITY;
     }
+    if (threadIdx.x < P.top && blockIdx.x == 0 && jj == 0) P.ew[(long long)b * P.ld_top + threadIdx.x] = mine / sum;
+    if (threadIdx.x == 0 && blockIdx.x == 0 && jj == 0 && P.Fs > 0) P.sgate[b] = sigmoidf(row[P.off_sg]);
+  } else {
+    if (threadIdx.x == 0) {
+      route_row(P, row, ids, val);
+      if (blockIdx.x == 0 && jj == 0) {
+        for (int q = 0; q < P.top; ++q) {
+          P.eids[(long long)b * P.ld_top + q] = ids[q];
+          P.ew[(long long)b * P.ld_top + q] = val[q];
+        }
+        if (P.Fs > 0) P.sgate[b] = sigmoidf(row[P.off_sg]);
+      }
+    }
+    __syncthreads();
+    e = ids[jj];
   }
-  __syncthreads();
   if (f >= P.F) return;
-  const int e = ids[jj];
   const T* x = (const T*)P.h + (long long)b * P.E;
   const T* wg = (const T*)P.w_gu + ((long long)e * 2 * P.F + f) * P.E;
   const T* wu = wg + (long long)P.F * P.E;

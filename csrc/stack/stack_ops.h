@@ -96,7 +96,8 @@ struct RetParams {
 };
 // rows of one sequence are contiguous and in position order; each sequence's state advances through them
 void retention(const RetParams& P, const StepRows& R, hipStream_t s);
-bool retention_supported(int D, int Dv);
+bool retention_supported(int D, int Dv);          // the state-in-registers kernel covers these head sizes
+bool retention_general_supported(int D, int Dv);  // the state-in-memory kernel covers the rest, up to 1024
 // the same recurrence in chunks (prompt portions), chunks in parallel around a scan over each sequence's chunk
 // states; `chunks` is a device table the host builds from the step's rows: per chunk {first row, rows (at most
 // retention_chunk_rows()), state slot, flags (1 = first chunk of its sequence's rows, 2 = last)}, a sequence's

@@ -50,6 +50,7 @@ MECHANISMS = {
     "retention": [(bc.ret(), None)],
     "retention_full_rot": [(bc.ret(heads=3, dim=8, vdim=8, decay=(0.5, 0.97, 0.9995), rot_dims=8), None)],
     "retention_no_rot": [(bc.ret(heads=1, dim=24, vdim=72, decay=(0.99,), rot_dims=0), None)],
+    "retention_wide_heads": [(bc.ret(heads=1, dim=72, vdim=264, decay=(0.98,), rot_dims=36), None)],
     "moe": [(bc.attn(heads=1, kv_heads=1, dim=8, vdim=8), bc.moe())],
     "moe_top1_no_shared": [(bc.attn(heads=1, kv_heads=1, dim=8, vdim=8), bc.moe(experts=5, top=1, ff=12, shared_ff=0))],
     "moe_all_experts": [(bc.ret(heads=1, dim=8, vdim=8, decay=(0.9,)), bc.moe(experts=3, top=3, ff=8, shared_ff=8))],
