@@ -140,6 +140,8 @@ PYBIND11_MODULE(_stack, m) {
         w.ld_top = geti(d, "ld_top");
         w.sgate = Pp<float>(ptr(d, "sgate"));
         w.lrows = Pp<void>(ptr(d, "lrows"));
+        w.split_ws = Pp<float>(ptr(d, "split_ws"));
+        w.split_ws_floats = d.contains("split_ws_floats") ? d["split_ws_floats"].cast<long long>() : 0;
         w.ret.chunks = Pp<const int>(ptr(d, "ret_chunks"));
         w.ret.max_chunks = geti(d, "ret_max_chunks");
         w.ret.U = Pp<float>(ptr(d, "ret_u"));
@@ -181,6 +183,10 @@ PYBIND11_MODULE(_stack, m) {
       .def("set_tiles", [](StackExecutor& e, int n) {
         if (n < 0 || n > e.max_tiles) throw std::runtime_error("stack executor: tile count outside the table");
         e.n_tiles = n;
+      })
+      .def("set_splits", [](StackExecutor& e, int n) {
+        if (n < 1 || n > 64) throw std::runtime_error("stack executor: splits outside 1..64");
+        e.n_splits = n;
       })
       .def("set_chunks", [](StackExecutor& e, int n) {
         if (n < 0 || n > e.ws.ret.max_chunks) throw std::runtime_error("stack executor: chunk count outside the table");

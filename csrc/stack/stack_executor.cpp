@@ -53,7 +53,7 @@ void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
   }
   StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
   AttnParams A{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.softcap,
-               L.qtemp_coef, L.qtemp_every, r.kc, r.vc, ws.a, ws.ld_a, f32};
+               L.qtemp_coef, L.qtemp_every, r.kc, r.vc, ws.a, ws.ld_a, f32, n_splits, ws.split_ws, ws.split_ws_floats};
   const bool fused_in = gemv_ln_supported(B, E, f32);
   if (fused_in) {  // decode steps: norm + input projection (+ query temperature and K/V store) in one launch
     gemv_ln(ws.resid, E, L.norm_w, L.norm_b, cfg.eps, L.w_in, B, L.n_in, ws.proj, ws.ld_proj, ws.h, L.kind == 0 ? &A : nullptr,

@@ -63,6 +63,8 @@ struct StackWorkspace {
   int ld_top = 0;
   float* sgate = nullptr;
   void* lrows = nullptr;   // [max_B][E] matrix dtype: normed rows for the head
+  float* split_ws = nullptr;  // decode attention over long contexts: per-split partials
+  long long split_ws_floats = 0;
   MoeGroupWs moe{};        // grouped routed feed-forward (prompt portions, bfloat16); gu == null: unused
   RetChunkWs ret{};        // chunked retention (prompt portions): chunk table, per-chunk states, o before its norm
 };
@@ -96,6 +98,7 @@ class StackExecutor {
   StackInputs in;
   const int* tiles = nullptr;  // attention query tiles of the NEXT step {first row, rows}, n_tiles of them (0: none)
   int n_tiles = 0, max_tiles = 0;
+  int n_splits = 1;        // blocks per (row, head) of the NEXT steps' decode attention (long contexts)
   int n_chunks = 0;        // chunks in ws.ret.chunks for the NEXT step (0: none bound, retention runs token by token)
 
   void validate() const;  // throws when a size does not fit the kernels or a pointer is missing

@@ -169,6 +169,8 @@ struct QkvEpi {
 };
 constexpr int LN_LDS_BYTES = 32768;
 constexpr int LN_RW = 4;  // weight rows per wave
+constexpr int LN_XR = 16;  // row elements per thread: E <= 4096
+constexpr int LN_PF = 4;  // 512-element steps of them requested before the norm (bfloat16)
 template <typename T>
 __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ x, int E, const float* __restrict__ nw,
                                                       const float* __restrict__ nb, float eps, const T* __restrict__ W,
@@ -178,25 +180,51 @@ __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ 
   __shared__ float red[4];
   T* hs = (T*)hs_raw;
   const int tid = threadIdx.x, lane = tid & 63;
-  for (int m = 0; m < M; ++m) {
+  const int n0 = (blockIdx.x * 4 + (tid >> 6)) * LN_RW;
+  // bfloat16: the first LN_PF steps of this wave's weight rows are requested before the norm, so the norm's round
+  // trips and barriers pass while the weights are on their way (E <= 2048: all of them)
+  constexpr bool PREF = sizeof(T) == 2;
+  u32x4 pre[LN_PF][LN_RW];
+  if (PREF && vec) {
+#pragma unroll
+    for (int it = 0; it < LN_PF; ++it)
+#pragma unroll
+      for (int u = 0; u < LN_RW; ++u) {
+        const int k = min(lane * 8 + it * 512, E - 8);
+        pre[it][u] = *(const u32x4*)(W + (long long)min(n0 + u, N - 1) * E + k);
+      }
+  }
+  for (int m = 0; m < M; ++m) {  // the row is read once (E <= 256 LN_XR) and normalised from registers
     const float* row = x + (long long)m * E;
+    float xr[LN_XR], gw[LN_XR], gb[LN_XR];
     float sum = 0.f;
-    for (int i = tid; i < E; i += 256) sum += row[i];
+#pragma unroll
+    for (int j = 0; j < LN_XR; ++j) {
+      const int i = tid + 256 * j;
+      xr[j] = i < E ? row[i] : 0.f;
+      gw[j] = i < E ? nw[i] : 0.f;
+      gb[j] = i < E ? nb[i] : 0.f;
+      sum += xr[j];
+    }
     const float mean = block_sum256(sum, red) / (float)E;
     float sq = 0.f;
-    for (int i = tid; i < E; i += 256) {
-      const float d = row[i] - mean;
+#pragma unroll
+    for (int j = 0; j < LN_XR; ++j) {
+      const float d = tid + 256 * j < E ? xr[j] - mean : 0.f;
       sq += d * d;
     }
     const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)E + eps);
-    for (int i = tid; i < E; i += 256) {
-      st(hs + (long long)m * E + i, (row[i] - mean) * rstd * nw[i] + nb[i]);
-      if (blockIdx.x == 0) hout[(long long)m * E + i] = hs[(long long)m * E + i];
+#pragma unroll
+    for (int j = 0; j < LN_XR; ++j) {
+      const int i = tid + 256 * j;
+      if (i < E) {
+        st(hs + (long long)m * E + i, (xr[j] - mean) * rstd * gw[j] + gb[j]);
+        if (blockIdx.x == 0) hout[(long long)m * E + i] = hs[(long long)m * E + i];
+      }
     }
   }
   __syncthreads();
   // LN_RW weight rows per wave, streamed together (independent loads in flight), against every activation row
-  const int n0 = (blockIdx.x * 4 + (tid >> 6)) * LN_RW;
   if (n0 >= N) return;
   for (int m = 0; m < M; ++m) {
     float accs[LN_RW];
@@ -205,7 +233,24 @@ __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ 
     const T* xr = hs + (long long)m * E;
     if (vec) {
       constexpr int PER = 16 / (int)sizeof(T);
-      for (int k = lane * PER; k < E; k += 64 * PER) {
+      int k = lane * PER;
+      if constexpr (PREF) {  // the steps fetched ahead
+#pragma unroll
+        for (int it = 0; it < LN_PF; ++it) {
+          if (k < E) {
+            float xv[8];
+            load8<T>(xr + k, xv);
+#pragma unroll
+            for (int u = 0; u < LN_RW; ++u)
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                accs[u] += __uint_as_float(pre[it][u][i] << 16) * xv[2 * i] +
+                           __uint_as_float(pre[it][u][i] & 0xffff0000u) * xv[2 * i + 1];
+          }
+          k += 64 * PER;
+        }
+      }
+      for (; k < E; k += 64 * PER) {
         float xv[8], wv[LN_RW][8];
 #pragma unroll
         for (int u = 0; u < LN_RW; ++u) {
@@ -260,7 +305,9 @@ __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ 
     }
   }
 }
-bool gemv_ln_supported(int M, int E, int f32) { return M > 0 && M <= 8 && (long long)M * E * (f32 ? 4 : 2) <= LN_LDS_BYTES; }
+bool gemv_ln_supported(int M, int E, int f32) {
+  return M > 0 && M <= 8 && E <= 256 * LN_XR && (long long)M * E * (f32 ? 4 : 2) <= LN_LDS_BYTES;
+}
 void gemv_ln(const float* x, int E, const float* nw, const float* nb, float eps, const void* W, int M, int N, float* C,
              int ldc, void* hout, const AttnParams* A, const StepRows* R, int f32, hipStream_t s) {
   check(gemv_ln_supported(M, E, f32) && x && nw && nb && W && C && hout && N > 0 && ldc >= N, "gemv_ln: bad operands");
@@ -779,7 +826,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
 // (weights and row indices come from LDS), so a group costs 16 short iterations instead of 64, and the four
 // quarters meet in two lane exchanges. The serial instruction count per wave is what bounds a decode step.
 template <typename T, int DPL>
-__global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, StepRows R, int vec, int vvec) {
+__global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, StepRows R, int vec, int vvec, int nsplit) {
   __shared__ __attribute__((aligned(16))) float qs[ATT_MAXD];
   __shared__ float ps[4][64];
   __shared__ int rs[4][64];
@@ -788,6 +835,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int b = blockIdx.x / P.H, h = blockIdx.x % P.H;
   const int g = h / (P.H / P.G);
+  const int split = blockIdx.y;  // long contexts: blockIdx.y-th of nsplit blocks, 64-key groups dealt round robin
   for (int d = threadIdx.x; d < P.D; d += 256) qs[d] = P.proj[(long long)b * P.ld + P.off_q + h * P.D + d];
   const int n = R.q_len[b];
   const int* bt = R.block_table + (long long)R.q_seq[b] * R.max_blocks;
@@ -798,7 +846,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
 #pragma unroll
   for (int c = 0; c < DPL; ++c) acc[c] = 0.f;
   __syncthreads();
-  for (int t0 = 64 * wv; t0 < n; t0 += 256) {
+  for (int t0 = 64 * (split * 4 + wv); t0 < n; t0 += 256 * nsplit) {
     const int t = t0 + lane;
     const bool valid = t < n;
     int rowidx = 0;
@@ -896,10 +944,23 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
 #pragma unroll
   for (int c = 0; c < DPL; ++c) acc[c] = 0.f;
   for (int w = 0; w < 4; ++w) {
-    const float f = expf(mg[w][0] - M);  // a wave without keys: exp(-inf) = 0
+    // a wave without keys has maximum -inf and weighs nothing; a block without keys (a short row beside a long
+    // one, split the same number of ways) has M = -inf too, and -inf - -inf must not become a NaN
+    const float f = mg[w][0] == -INFINITY ? 0.f : expf(mg[w][0] - M);
     L += mg[w][1] * f;
 #pragma unroll
     for (int c = 0; c < DPL; ++c) acc[c] += ag[w][dq * DPL + c] * f;
+  }
+  if (nsplit > 1) {  // partial {maximum, sum, un-normalised output}; attention_merge_kernel finishes the row
+    float* w = P.split_ws + ((long long)blockIdx.x * nsplit + split) * (P.Dv + 2);
+    if (lane == 0) {
+      w[0] = M;
+      w[1] = L;
+    }
+#pragma unroll
+    for (int c = 0; c < DPL; ++c)
+      if (dq * DPL + c < P.Dv) w[2 + dq * DPL + c] = acc[c];
+    return;
   }
   T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
   const float inv = 1.f / L;
@@ -907,21 +968,48 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
   for (int c = 0; c < DPL; ++c)
     if (dq * DPL + c < P.Dv) st(out + dq * DPL + c, acc[c] * inv);
 }
+// one wave per (row, head): the nsplit partials of a long context into the output
+template <typename T>
+__global__ __launch_bounds__(256) void attention_merge_kernel(AttnParams P, int items, int nsplit) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= items) return;
+  const float* w = P.split_ws + (long long)item * nsplit * (P.Dv + 2);
+  float M = -INFINITY;
+  for (int sidx = 0; sidx < nsplit; ++sidx) M = fmaxf(M, w[(long long)sidx * (P.Dv + 2)]);
+  float L = 0.f;
+  for (int sidx = 0; sidx < nsplit; ++sidx) {
+    const float ms = w[(long long)sidx * (P.Dv + 2)];
+    if (ms != -INFINITY) L += w[(long long)sidx * (P.Dv + 2) + 1] * expf(ms - M);  // a split without keys weighs nothing
+  }
+  T* out = (T*)P.out + (long long)(item / P.H) * P.ld_out + (item % P.H) * P.Dv;
+  for (int d = lane; d < P.Dv; d += 64) {
+    float o = 0.f;
+    for (int sidx = 0; sidx < nsplit; ++sidx) {
+      const float ms = w[(long long)sidx * (P.Dv + 2)];
+      if (ms != -INFINITY) o += w[(long long)sidx * (P.Dv + 2) + 2 + d] * expf(ms - M);
+    }
+    st(out + d, o / L);
+  }
+}
 template <typename T>
 static void launch_attention_decode(const AttnParams& P, const StepRows& R, hipStream_t s) {
   const int vec = P.D % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
-  dim3 grid(R.B * P.H);
+  const int ns = (P.nsplit > 1 && P.split_ws && (long long)R.B * P.H * P.nsplit * (P.Dv + 2) <= P.split_ws_floats) ? P.nsplit : 1;
+  dim3 grid(R.B * P.H, ns);
   const int per = 16 / (int)sizeof(T);  // elements of a 16-byte load
   if (P.Dv <= 64) {
     const int vvec = P.Dv % 4 == 0 && (sizeof(T) == 2 ? 1 : 0) && ((uintptr_t)P.vc & 15) == 0;  // 8-byte pieces (bf16)
-    hipLaunchKernelGGL((attention_decode_kernel<T, 4>), grid, dim3(256), 0, s, P, R, vec, sizeof(T) == 2 ? vvec : 0);
+    hipLaunchKernelGGL((attention_decode_kernel<T, 4>), grid, dim3(256), 0, s, P, R, vec, sizeof(T) == 2 ? vvec : 0, ns);
   } else if (P.Dv <= 128) {
     const int vvec = P.Dv % 8 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
-    hipLaunchKernelGGL((attention_decode_kernel<T, 8>), grid, dim3(256), 0, s, P, R, vec, vvec);
+    hipLaunchKernelGGL((attention_decode_kernel<T, 8>), grid, dim3(256), 0, s, P, R, vec, vvec, ns);
   } else {
     const int vvec = P.Dv % 16 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
-    hipLaunchKernelGGL((attention_decode_kernel<T, 16>), grid, dim3(256), 0, s, P, R, vec, vvec);
+    hipLaunchKernelGGL((attention_decode_kernel<T, 16>), grid, dim3(256), 0, s, P, R, vec, vvec, ns);
   }
+  if (ns > 1)
+    hipLaunchKernelGGL(attention_merge_kernel<T>, dim3((R.B * P.H + 3) / 4), dim3(256), 0, s, P, R.B * P.H, ns);
 }
 
 template <typename T, int RQ, int DC>
@@ -1764,7 +1852,8 @@ __global__ __launch_bounds__(256) void moe_route_experts_kernel(MoeParams P, int
     e = 0;
     for (int q = 0; q < P.top; ++q) {
       const float mx = wave_max(z);
-      const int who = __ffsll((unsigned long long)__ballot(z == mx)) - 1;
+      // non-finite logits (a fault upstream) compare unequal to everything: expert 0 then, never an index of -1
+      const int who = max(0, __ffsll((unsigned long long)__ballot(z == mx)) - 1);
       if (q == 0) mx0 = mx;
       const float w = expf(mx - mx0);
       sum += w;

@@ -62,6 +62,11 @@ struct AttnParams {
   void* out;            // [B][ld_out] matrix dtype, head-major
   int ld_out;
   int f32;
+  // decode steps over long contexts: nsplit blocks per (row, head) share the keys and leave partials
+  // {maximum, sum, output} in split_ws, a second launch merges them (nsplit <= 1: one block finishes the row)
+  int nsplit;
+  float* split_ws;
+  long long split_ws_floats;
 };
 // q *= 1 + coef * ln(floor((pos + 1) / every) + 1); k, v of every row stored at its slot
 void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s);

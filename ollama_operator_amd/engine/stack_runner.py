@@ -63,6 +63,7 @@ class StackExec:
                              ld_proj=r.proj.shape[1], a=p(r.abuf), ld_a=r.abuf.shape[1], hmid=p(r.hmid),
                              ld_hmid=r.hmid.shape[1], y=p(r.ybuf), eids=p(r.eids), ew=p(r.ew), ld_top=r.eids.shape[1],
                              sgate=p(r.sgate), lrows=p(r.lbuf), obuf=p(r.obuf), ld_obuf=r.obuf.shape[1],
+                             split_ws=p(r.split_ws), split_ws_floats=r.split_ws.numel(),
                              ret_chunks=p(r.d_chunks), ret_max_chunks=r.d_chunks.shape[0], ret_u=p(r.ret_u),
                              ret_sin=p(r.ret_sin), ret_u_stride=r.ret_u.shape[1],
                              **{"moe_" + k: (v if isinstance(v, int) else p(v)) for k, v in r.moe_ws.items()}))
@@ -105,7 +106,12 @@ class StackExec:
     def run(self, stage: str, layer: int, B: int, n_logits: int = 0, use_idx: bool = False, prefill: bool = False):
         if stage in ("forward", "embed"):  # a new step: its rows as the host uploaded them, if it did
             rows, self.r._step_rows = self.r._step_rows, None
-            self.bind_chunks(rows if rows is not None and len(rows[0]) == B else None)
+            rows = rows if rows is not None and len(rows[0]) == B else None
+            self.bind_chunks(rows)
+            # decode attention: blocks per (row, head) by the longest context of the step. A batch-1 step says
+            # it itself (`_decode_S`, part of its graph's key); other steps by the rows the host uploaded
+            S = self.r._decode_S or (self.r.decode_splits(max(rows[0]) + 1) if rows is not None else 1)
+            self.exe.set_splits(max(1, S))
         self.exe.step(self.stages[stage], layer, B, n_logits, use_idx, torch.cuda.current_stream().cuda_stream)
 
 
@@ -170,6 +176,9 @@ class StackRunner(Runner):
         self.d_tiles = torch.zeros(max_batch // 32 + max_seqs + 1, 2, **i32)  # attention query tiles of a step
         self.ret_u = torch.zeros(n_ch, max([m.heads * m.dim * m.vdim for m in rets], default=1) if n_ch > 1 else 1, **f32)
         self.ret_sin = torch.zeros_like(self.ret_u)
+        # decode attention over long contexts: partials {maximum, sum, output} of up to 16 splits per (row, head)
+        hv = max([s.mixer.heads * (s.mixer.vdim + 2) for s in cfg.layers if s.mixer.kind == MIX_ATTENTION], default=1)
+        self.split_ws = torch.zeros(16 * 16 * hv, **f32)
         self._step_rows = None  # (positions, sequence rows) of the rows last uploaded, until a step consumes them
         # routed feed-forward of prompt portions (bfloat16): pairs sorted by expert, per-expert matrix-core products
         self.moe_ws = {}
@@ -219,6 +228,14 @@ class StackRunner(Runner):
 
     def split_plan(self, B: int) -> tuple[int, int]:
         return 1, 0
+
+    def decode_splits(self, length: int) -> int:
+        """Blocks per (row, head) of the decode attention over `length` keys: 1 up to 512 keys, then a power of
+        two with about 256 keys per block, at most 16. Batch-1 decode graphs are captured per bucket."""
+        S = 1
+        while S < 16 and length > 256 * S * 2:
+            S *= 2
+        return S
 
     def _output_norm(self, h: torch.Tensor) -> torch.Tensor:
         return torch.nn.functional.layer_norm(h, (h.shape[-1],), self.w.final_w, self.w.final_b, self.cfg.norm_eps)
@@ -272,8 +289,11 @@ class StackRunner(Runner):
                 self.prefill(sid, [(i * 7919 + 3) % V for i in range(n)])
             finally:
                 self.free_sequence(sid)
-        if self.use_graphs:
-            self._graph(1)
+        if self.use_graphs:  # one batch-1 decode graph per attention split bucket reachable at this context
+            for S in sorted({self.decode_splits(n) for n in (1, 513, 1025, 2049, 4097, 8193) if n <= self.ctx}):
+                self._decode_S = S
+                self._graph(1)
+            self._decode_S = 0
         torch.cuda.synchronize()
 
 

@@ -219,6 +219,34 @@ def test_one_key_stands_out(tmp_path, device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_long_context_decode(tmp_path, device):
+    """Single tokens after 1300 and after 2300 cached keys: on a GPU the decode attention then shares a row's keys
+    among several blocks and merges their partial softmax sums; sharp scores make single far keys matter."""
+    layers = [(bc.attn(heads=4, kv_heads=2, dim=16, vdim=24, scale=1.5, softcap=40.0, coef=0.5, every=512), None),
+              (bc.attn(heads=2, kv_heads=1, dim=64, vdim=64, scale=0.4, softcap=0.0, coef=0.0), None)]
+    m = bc.Model(tmp_path, bc.config(layers, width=32, vocab=60, mult=1.0, cap=0.0), seed=21)
+    toks = bc.tokens(2306, 60, seed=22)
+    want, _ = m.oracle(toks)
+    r = m.runner(device, max_batch=512, kv_tokens=2400)
+    cuts = [1300, 1301, 1302, 1303, 2300] + list(range(2301, 2307))
+    got = bc.run_cuts(r, toks, cuts)
+    rows = [1300, 1301, 1302] + list(range(2300, 2306))
+    bc.check(got[rows], want[rows], "float32", "decoded after a long context")
+    # a long sequence's single token beside a short sequence's two: the short rows' extra blocks have no keys
+    short = bc.tokens(9, 60, seed=23)
+    ws = m.oracle(short)[0]
+    a, b = r.new_sequence(), r.new_sequence()
+    r.step_entries([(a, toks[:2200], []), (b, short[:5], [])])
+    out = r.step_entries([(a, toks[2200:2201], [0]), (b, short[5:7], [0, 1])]).float().cpu().numpy()
+    bc.check(out[:1], want[2200:2201], "float32", "long row of a mixed step")
+    bc.check(out[1:], ws[5:7], "float32", "short rows of a mixed step")
+    r2 = m.runner(device, "bfloat16", max_batch=512, kv_tokens=2400, use_graphs=None)
+    sid = r2.new_sequence()
+    out = list(r2.generate(sid, toks[:1100], SamplingOptions(temperature=0.0, repeat_penalty=1.0), max_tokens=3))
+    assert len(out) == 3  # the batch-1 decode graph of a split bucket runs
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_first_tokens(std, device):
     for n in (1, 2, 3):
         toks = bc.tokens(n, 96, seed=50 + n)
