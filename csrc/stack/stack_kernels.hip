@@ -1107,35 +1107,53 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   const float inv_cap = P.softcap != 0.f ? 1.f / P.softcap : 0.f;
   const uint16_t* kc = (const uint16_t*)P.kc;
   const uint16_t* vc = (const uint16_t*)P.vc;
-  for (int t0 = 0; t0 < kmax; t0 += 32) {
-    // V rows of this key group into LDS (keys past the end: the last key's row, their weights are zero)
-    __syncthreads();
-    {
-      constexpr int CH = DV / 8;  // 16-byte pieces per row
-#pragma unroll
-      for (int c = lane; c < 32 * CH; c += 64) {
-        const int key = min(t0 + c / CH, kmax - 1), seg = c % CH;
-        const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
-        const u32x4 v = *(const u32x4*)(vc + rowidx * DV + 8 * seg);
-        unsigned* dst = (unsigned*)&Vl[(c / CH) * LDV + 8 * seg];
-        *(unsigned long long*)dst = (unsigned long long)v[0] | ((unsigned long long)v[1] << 32);
-        *(unsigned long long*)(dst + 2) = (unsigned long long)v[2] | ((unsigned long long)v[3] << 32);
-      }
-    }
-    // S^T = K Q^T
-    f32x16 sacc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+  // The K fragments and V rows of the NEXT key group are requested before the current group is multiplied, so a
+  // group's global round trip passes behind the previous group's products and softmax.
+  constexpr int CH = DV / 8;            // 16-byte pieces per V row
+  constexpr int VPL = 32 * CH / 64;     // V pieces per lane per group
+  u32x4 kf_n[KD], vs_n[VPL];
+  auto fetch = [&](int t0) {
     {
       const int key = min(t0 + kperm, kmax - 1);
       const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
       const uint16_t* kr = kc + rowidx * D + 8 * hf;
 #pragma unroll
-      for (int kk = 0; kk < KD; ++kk) {
-        const bf16x8 kf = __builtin_bit_cast(bf16x8, *(const u32x4*)(kr + 16 * kk));
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qhi[kk], sacc, 0, 0, 0);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qlo[kk], sacc, 0, 0, 0);
-      }
+      for (int kk = 0; kk < KD; ++kk) kf_n[kk] = *(const u32x4*)(kr + 16 * kk);
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {  // keys past the end: the last key's row, their weights are zero
+      const int c = lane + 64 * i;
+      const int key = min(t0 + c / CH, kmax - 1), seg = c % CH;
+      const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
+      vs_n[i] = *(const u32x4*)(vc + rowidx * DV + 8 * seg);
+    }
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < kmax; t0 += 32) {
+    u32x4 kf_c[KD], vs_c[VPL];
+#pragma unroll
+    for (int kk = 0; kk < KD; ++kk) kf_c[kk] = kf_n[kk];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) vs_c[i] = vs_n[i];
+    if (t0 + 32 < kmax) fetch(t0 + 32);
+    // V rows of this key group into LDS
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int c = lane + 64 * i;
+      unsigned* dst = (unsigned*)&Vl[(c / CH) * LDV + 8 * (c % CH)];
+      *(unsigned long long*)dst = (unsigned long long)vs_c[i][0] | ((unsigned long long)vs_c[i][1] << 32);
+      *(unsigned long long*)(dst + 2) = (unsigned long long)vs_c[i][2] | ((unsigned long long)vs_c[i][3] << 32);
+    }
+    // S^T = K Q^T
+    f32x16 sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KD; ++kk) {
+      const bf16x8 kf = __builtin_bit_cast(bf16x8, kf_c[kk]);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qhi[kk], sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qlo[kk], sacc, 0, 0, 0);
     }
     // register r of lane (q, hf) is key t0 + 16 (r >> 3) + 8 hf + (r & 7)
     float pr[16];
