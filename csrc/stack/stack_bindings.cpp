@@ -48,6 +48,8 @@ PYBIND11_MODULE(_stack, m) {
   m.def("gemm_path", &gemm_path);
   m.def("set_gemm_mfma", &set_gemm_mfma);
   m.def("retention_supported", &retention_supported);
+  m.def("gated_scan_supported", &gated_scan_supported);
+  m.def("latent_supported", &latent_supported);
   m.def("retention_chunk_rows", &retention_chunk_rows);
   m.attr("FLASH_TILE_ROWS") = (int)FLASH_TILE_ROWS;
 
@@ -62,6 +64,8 @@ PYBIND11_MODULE(_stack, m) {
         e.cfg.f32 = geti(c, "f32");
         e.cfg.max_B = geti(c, "max_B");
         e.cfg.max_seqs = geti(c, "max_seqs");
+        e.cfg.block = geti(c, "block");
+        e.cfg.embed_scale = getf(c, "embed_scale", 1.f);
       })
       .def("set_globals", [](StackExecutor& e, py::dict d) {
         e.embed_w = Pp<const void>(ptr(d, "embed"));
@@ -108,6 +112,39 @@ PYBIND11_MODULE(_stack, m) {
         L.w_gu = Pp<const void>(ptr(d, "w_gu"));
         L.w_down = Pp<const void>(ptr(d, "w_down"));
         L.sh_down = Pp<const void>(ptr(d, "sh_down"));
+        L.norm2_w = Pp<const float>(ptr(d, "norm2_w"));
+        L.norm2_b = Pp<const float>(ptr(d, "norm2_b"));
+        L.w_ff = Pp<const void>(ptr(d, "w_ff"));
+        L.n_ff = geti(d, "n_ff");
+        L.ff_dense = geti(d, "ff_dense");
+        L.w_dense_down = Pp<const void>(ptr(d, "w_dense_down"));
+        L.identity = geti(d, "identity");
+        L.group_count = geti(d, "group_count", 1);
+        L.group_keep = geti(d, "group_keep", 1);
+        L.rot_dim = geti(d, "rot_dim");
+        L.kv_rank = geti(d, "kv_rank");
+        L.inv_freq64 = Pp<const double>(ptr(d, "inv_freq64"));
+        L.dkv_norm = Pp<const float>(ptr(d, "dkv_norm"));
+        L.w_uk = Pp<const void>(ptr(d, "w_uk"));
+        L.w_uvT = Pp<const void>(ptr(d, "w_uvT"));
+        L.sink = Pp<const float>(ptr(d, "sink"));
+        L.gate_cap = getf(d, "gate_cap");
+        L.off_i = geti(d, "off_i");
+        L.off_f = geti(d, "off_f");
+        L.i_b = Pp<const float>(ptr(d, "i_b"));
+        L.f_b = Pp<const float>(ptr(d, "f_b"));
+        L.mnorm = Pp<const float>(ptr(d, "mnorm"));
+        L.state = geti(d, "state");
+        L.groups = geti(d, "groups", 1);
+        L.conv = geti(d, "conv", 1);
+        L.norm_groups = geti(d, "norm_groups", 1);
+        L.off_conv = geti(d, "off_conv");
+        L.off_dt = geti(d, "off_dt");
+        L.conv_w = Pp<const float>(ptr(d, "conv_w"));
+        L.conv_b = Pp<const float>(ptr(d, "conv_b"));
+        L.dt_bias = Pp<const float>(ptr(d, "dt_bias"));
+        L.a_log = Pp<const float>(ptr(d, "a_log"));
+        L.d_skip = Pp<const float>(ptr(d, "d_skip"));
         if (L.qtemp_every <= 0) throw std::runtime_error("q_temp.every must be positive");
       })
       .def("set_runs", [](StackExecutor& e, std::vector<py::dict> runs) {
@@ -119,6 +156,7 @@ PYBIND11_MODULE(_stack, m) {
           r.kc = Pp<void>(ptr(d, "kc"));
           r.vc = Pp<void>(ptr(d, "vc"));
           r.state = Pp<float>(ptr(d, "state"));
+          r.state_stride = d.contains("state_stride") ? d["state_stride"].cast<long long>() : 0;
           e.runs.push_back(r);
         }
       })
@@ -159,6 +197,11 @@ PYBIND11_MODULE(_stack, m) {
         w.moe.max_pairs = geti(d, "moe_max_pairs");
         w.moe.max_tiles = geti(d, "moe_max_tiles");
         w.ret.ld_o = geti(d, "ld_obuf");
+        w.cbuf = Pp<float>(ptr(d, "cbuf"));
+        w.ld_cbuf = geti(d, "ld_cbuf");
+        w.lat = Pp<void>(ptr(d, "lat"));
+        w.ld_lat = geti(d, "ld_lat");
+        w.idw = Pp<float>(ptr(d, "idw"));
       })
       .def("set_inputs", [](StackExecutor& e, py::dict d) {
         StackInputs& in = e.in;

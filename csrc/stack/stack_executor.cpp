@@ -10,6 +10,38 @@ static void need(bool ok, const std::string& what) {
   if (!ok) throw std::runtime_error("stack executor: " + what);
 }
 
+static void validate_postnorm(const StackExecutor& e, const RunDesc& r, const LayerDesc& L) {
+  const StackWorkspace& ws = e.ws;
+  need(L.kind >= 2 && L.kind <= 4, "a layer with output norms needs a latent attention, mLSTM or Mamba-2 mixer");
+  need(ws.ret.ld_o >= L.heads * L.vdim && ws.ret.obuf, "mixer output wider than its float32 buffer");
+  if (L.kind == 2) {
+    need(r.kc && L.w_uk && L.w_uvT && L.dkv_norm && L.sink && ws.cbuf && ws.lat, "latent attention operands");
+    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim), "latent attention sizes (dim <= 256, kv_rank + rot_dim <= 256)");
+    need(L.heads * (L.kv_rank + L.rot_dim) <= ws.ld_cbuf && L.heads * L.kv_rank <= ws.ld_lat, "latent attention buffers");
+    need(L.rot_dims == 0 || L.inv_freq64, "latent attention rotary table missing");
+  } else if (L.kind == 3) {
+    need(r.state && L.i_b && L.f_b && L.mnorm && L.gate_cap > 0.f, "mLSTM operands");
+    need(gated_scan_supported(SCAN_MLSTM, L.dim, L.vdim), "mLSTM head sizes (dim <= 256, vdim <= 255, dim * (vdim + 1) <= 16384)");
+    need(r.state_stride >= (long long)L.heads * (L.dim * L.vdim + L.dim + 1), "mLSTM state slot too small");
+  } else {
+    need(r.state && L.conv_w && L.conv_b && L.dt_bias && L.a_log && L.d_skip && L.mnorm && ws.cbuf, "Mamba-2 operands");
+    need(gated_scan_supported(SCAN_SSD, L.state, L.vdim), "Mamba-2 head sizes (state <= 256, vdim <= 256, state * vdim <= 16384)");
+    const long long ch = (long long)L.heads * L.vdim + 2LL * L.groups * L.state;
+    need(ch <= ws.ld_cbuf && L.groups > 0 && L.heads % L.groups == 0 && L.conv >= 1, "Mamba-2 convolution sizes");
+    need(r.state_stride >= (long long)L.heads * L.state * L.vdim + (L.conv - 1) * ch, "Mamba-2 state slot too small");
+    need(L.norm_groups > 0 && (L.heads * L.vdim) % L.norm_groups == 0, "Mamba-2 norm groups");
+  }
+  if (L.ff_dense) {
+    need(L.w_ff && L.w_dense_down && L.norm2_w && L.norm2_b && L.ff > 0 && L.ff <= ws.ld_hmid && L.ff <= ws.ld_proj && ws.hmid,
+         "dense feed-forward operands");
+  } else if (L.experts) {
+    need(L.w_ff && L.norm2_w && L.norm2_b && L.n_ff <= ws.ld_proj && L.top > 0 && L.top <= MOE_MAX_TOP && L.top <= ws.ld_top &&
+             L.top * L.ff + L.shared_ff <= ws.ld_hmid && ws.hmid && ws.eids && ws.ew && ws.idw && L.router_b && L.w_gu &&
+             L.w_down && (!L.shared_ff || (L.sh_down && ws.sgate)),
+         "routed feed-forward operands");
+  }
+}
+
 void StackExecutor::validate() const {
   need(cfg.E > 0 && cfg.V > 0 && cfg.max_B > 0, "not configured");
   need(embed_w && final_w && final_b && head_w, "global weights missing");
@@ -21,6 +53,10 @@ void StackExecutor::validate() const {
     const LayerDesc& L = layers[r.layer];
     need(L.norm_w && L.norm_b && L.w_in && L.w_o && L.n_in > 0 && L.n_in <= ws.ld_proj, "layer weights missing");
     need(L.heads * L.vdim <= ws.ld_a, "mixer output wider than its buffer");
+    if (cfg.block == 1) {
+      validate_postnorm(*this, r, L);
+      continue;
+    }
     if (r.opens_pass) need(loop_in && ws.cat, "the pass-opening projection is missing");
     if (L.kind == 0) {
       need(r.kc && r.vc, "attention run without a K/V pool");
@@ -39,10 +75,126 @@ void StackExecutor::validate() const {
 }
 
 void StackExecutor::embed(int B, hipStream_t s) {
-  stack::embed(embed_w, in.tokens, B, cfg.E, cfg.V, ws.resid, ws.x0, cfg.f32, s);
+  h_ready = false;
+  stack::embed(embed_w, in.tokens, B, cfg.E, cfg.V, ws.resid, ws.x0, cfg.embed_scale, cfg.f32, s);
+}
+
+// x <- x + LN1(mixer(x)), then x <- x + LN2(ff(x)): both sublayers read the stream itself (cast to the matrix
+// dtype), the layer norm sits on their outputs.
+void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
+  const RunDesc& r = runs.at(ri);
+  const LayerDesc& L = layers[r.layer];
+  const int E = cfg.E, f32 = cfg.f32, n_out = L.heads * L.vdim;
+  StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
+  if (!h_ready) cast_rows(ws.resid, B, E, ws.h, f32, s);  // else the previous update left the rows in ws.h
+  {  // every matrix of the mixer that reads the stream, in one product
+    GemmParams g{ws.h, E, L.w_in, B, L.n_in, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  if (L.kind == 2) {
+    const int C = L.kv_rank, W = C + L.rot_dim;
+    LatentParams P{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_g, L.heads, L.dim, L.rot_dim, C, L.vdim, L.rot_dims,
+                   L.inv_freq64, L.dkv_norm, cfg.eps, L.w_uk, L.w_uvT, r.kc, ws.cbuf, ws.ld_cbuf, ws.lat, ws.ld_lat, ws.a,
+                   ws.ld_a, f32};
+    latent_prepare(P, R, s);
+    // one cached row per token serves every head: attention with a single key/value head whose key is the whole
+    // row and whose value is the row's first C elements
+    AttnParams A{ws.cbuf, ws.ld_cbuf, 0, 0, 0, L.heads, 1, W, C, L.scale, 0.f, 0.f, 1, r.kc, r.kc, ws.lat, ws.ld_lat, f32,
+                 n_splits, ws.split_ws, ws.split_ws_floats, W, W, L.sink};
+    attention(A, R, s);
+    latent_expand(P, B, s);
+  } else if (L.kind == 3) {
+    ScanParams P{};
+    P.mode = SCAN_MLSTM;
+    P.proj = ws.proj;
+    P.ld = ws.ld_proj;
+    P.off_q = L.off_q;
+    P.off_k = L.off_k;
+    P.off_v = L.off_v;
+    P.off_i = L.off_i;
+    P.off_f = L.off_f;
+    P.H = P.G = L.heads;
+    P.D = L.dim;
+    P.Dv = L.vdim;
+    P.i_b = L.i_b;
+    P.f_b = L.f_b;
+    P.cap = L.gate_cap;
+    P.state = r.state;
+    P.state_stride = r.state_stride;
+    P.y = ws.ret.obuf;
+    P.ld_y = ws.ret.ld_o;
+    gated_scan(P, R, s);
+    // per-head unit RMS, the norm's weight, the sigmoid output gate
+    group_rms_cast(ws.ret.obuf, ws.ret.ld_o, B, n_out, L.heads, L.mnorm, cfg.eps, ws.proj + L.off_g, ws.ld_proj, ws.a, ws.ld_a, f32, s);
+  } else {
+    const int ch = n_out + 2 * L.groups * L.state;
+    ConvParams Cv{ws.proj, ws.ld_proj, L.off_conv, ch, L.conv, L.conv_w, L.conv_b,
+                  r.state + (long long)L.heads * L.state * L.vdim, r.state_stride, ws.cbuf, ws.ld_cbuf};
+    conv_silu(Cv, R, s);
+    ScanParams P{};
+    P.mode = SCAN_SSD;
+    P.proj = ws.proj;
+    P.ld = ws.ld_proj;
+    P.conv = ws.cbuf;
+    P.ld_conv = ws.ld_cbuf;
+    P.off_v = 0;                                  // x | B | C
+    P.off_k = n_out;
+    P.off_q = n_out + L.groups * L.state;
+    P.off_i = L.off_dt;
+    P.off_g = L.off_g;
+    P.H = L.heads;
+    P.G = L.groups;
+    P.D = L.state;
+    P.Dv = L.vdim;
+    P.dt_bias = L.dt_bias;
+    P.a_log = L.a_log;
+    P.d_skip = L.d_skip;
+    P.state = r.state;
+    P.state_stride = r.state_stride;
+    P.y = ws.ret.obuf;
+    P.ld_y = ws.ret.ld_o;
+    gated_scan(P, R, s);
+    group_rms_cast(ws.ret.obuf, ws.ret.ld_o, B, n_out, L.norm_groups, L.mnorm, cfg.eps, nullptr, 0, ws.a, ws.ld_a, f32, s);
+  }
+  {
+    GemmParams o{ws.a, ws.ld_a, L.w_o, B, E, n_out, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(o, s);
+  }
+  const bool has_ff = L.ff_dense || L.experts;
+  // the updated rows leave in the matrix dtype too: the next product's operand (feed-forward, or the next layer)
+  post_norm_add(ws.resid, ws.y, B, E, L.norm_w, L.norm_b, cfg.eps, nullptr, ws.h, f32, s);
+  h_ready = true;
+  if (!has_ff) return;
+  {
+    GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  const float* idw = nullptr;
+  if (L.ff_dense) {
+    relu2_cast(ws.proj, ws.ld_proj, B, L.ff, ws.hmid, ws.ld_hmid, f32, s);
+    GemmParams d{ws.hmid, ws.ld_hmid, L.w_dense_down, B, E, L.ff, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(d, s);
+  } else {
+    MoeParams M{ws.proj, ws.ld_proj, L.off_router, 0, L.off_sgate, L.off_sup, B, E, L.experts, L.top, L.ff, L.shared_ff,
+                L.router_b, ws.h, L.w_gu, L.w_down, L.sh_down, ws.eids, ws.ew, ws.ld_top, ws.sgate, ws.hmid, ws.ld_hmid, ws.y,
+                f32, L.identity, L.group_count, L.group_keep, ws.idw};
+    moe_route_scores(M, s);
+    if (B > SMALL_B && ws.moe.gu && moe_grouped_supported(M)) {
+      moe_grouped(M, ws.moe, s);
+    } else {
+      moe_experts(M, s);
+      moe_down(M, s);
+    }
+    if (L.identity) idw = ws.idw;
+  }
+  post_norm_add(ws.resid, ws.y, B, E, L.norm2_w, L.norm2_b, cfg.eps, idw, ws.h, f32, s);
 }
 
 void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
+  if (cfg.block == 1) {
+    layer_run_postnorm(ri, B, s);
+    return;
+  }
   const RunDesc& r = runs.at(ri);
   const LayerDesc& L = layers[r.layer];
   const int E = cfg.E, f32 = cfg.f32;

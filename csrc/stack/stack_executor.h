@@ -17,10 +17,12 @@ struct StackConfig {
   float eps = 1e-5f, residual_mult = 1.f, logit_softcap = 0.f;
   int f32 = 0;
   int max_B = 0, max_seqs = 0;
+  int block = 0;            // 0: one norm, mixer and feed-forward in parallel; 1: norms on the sublayers' outputs
+  float embed_scale = 1.f;
 };
 
 struct LayerDesc {
-  int kind = 0;  // 0 attention, 1 retention
+  int kind = 0;  // 0 attention, 1 retention, 2 latent attention, 3 mLSTM, 4 Mamba-2
   int heads = 0, kv_heads = 0, dim = 0, vdim = 0;
   float scale = 1.f, softcap = 0.f, qtemp_coef = 0.f;
   int qtemp_every = 1, rot_dims = 0;
@@ -36,6 +38,32 @@ struct LayerDesc {
   const void* w_gu = nullptr;
   const void* w_down = nullptr;
   const void* sh_down = nullptr;
+  // layers with norms on the sublayers' outputs
+  const float* norm2_w = nullptr;   // the feed-forward's output norm
+  const float* norm2_b = nullptr;
+  const void* w_ff = nullptr;       // [n_ff][E]: router | shared gate | shared up, or the dense up projection
+  int n_ff = 0;
+  int ff_dense = 0;                 // 1: W_down relu(W_up h)^2 with `ff` hidden units
+  const void* w_dense_down = nullptr;
+  int identity = 0, group_count = 1, group_keep = 1;  // score router
+  int rot_dim = 0, kv_rank = 0;     // latent attention
+  const double* inv_freq64 = nullptr;
+  const float* dkv_norm = nullptr;
+  const void* w_uk = nullptr;
+  const void* w_uvT = nullptr;
+  const float* sink = nullptr;
+  float gate_cap = 0.f;             // mLSTM
+  int off_i = 0, off_f = 0;
+  const float* i_b = nullptr;
+  const float* f_b = nullptr;
+  const float* mnorm = nullptr;     // weight of the mixer's own output norm (mLSTM, Mamba-2)
+  int state = 0, groups = 1, conv = 1, norm_groups = 1;  // Mamba-2
+  int off_conv = 0, off_dt = 0;
+  const float* conv_w = nullptr;
+  const float* conv_b = nullptr;
+  const float* dt_bias = nullptr;
+  const float* a_log = nullptr;
+  const float* d_skip = nullptr;
 };
 
 struct RunDesc {   // one execution of a layer: its own cache
@@ -44,6 +72,7 @@ struct RunDesc {   // one execution of a layer: its own cache
   void* kc = nullptr;
   void* vc = nullptr;
   float* state = nullptr;
+  long long state_stride = 0;  // floats per slot (mLSTM, Mamba-2: the slot's whole state)
 };
 
 struct StackWorkspace {
@@ -65,6 +94,11 @@ struct StackWorkspace {
   void* lrows = nullptr;   // [max_B][E] matrix dtype: normed rows for the head
   float* split_ws = nullptr;  // decode attention over long contexts: per-split partials
   long long split_ws_floats = 0;
+  float* cbuf = nullptr;   // [max_B][ld_cbuf] float32: latent attention's folded queries, the convolution's output
+  int ld_cbuf = 0;
+  void* lat = nullptr;     // [max_B][ld_lat] matrix dtype: attention outputs in latent space
+  int ld_lat = 0;
+  float* idw = nullptr;    // [max_B] weight of the chosen identity experts
   MoeGroupWs moe{};        // grouped routed feed-forward (prompt portions, bfloat16); gu == null: unused
   RetChunkWs ret{};        // chunked retention (prompt portions): chunk table, per-chunk states, o before its norm
 };
@@ -99,11 +133,13 @@ class StackExecutor {
   const int* tiles = nullptr;  // attention query tiles of the NEXT step {first row, rows}, n_tiles of them (0: none)
   int n_tiles = 0, max_tiles = 0;
   int n_splits = 1;        // blocks per (row, head) of the NEXT steps' decode attention (long contexts)
+  bool h_ready = false;    // ws.h holds the stream's rows in the matrix dtype (layers with output norms)
   int n_chunks = 0;        // chunks in ws.ret.chunks for the NEXT step (0: none bound, retention runs token by token)
 
   void validate() const;  // throws when a size does not fit the kernels or a pointer is missing
   void embed(int B, hipStream_t s);
   void layer_run(int ri, int B, hipStream_t s);
+  void layer_run_postnorm(int ri, int B, hipStream_t s);
   void head(int n_logits, bool use_idx, hipStream_t s);
   void forward(int B, int n_logits, bool use_idx, hipStream_t s);
 };

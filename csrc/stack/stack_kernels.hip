@@ -8,112 +8,11 @@
 #include <stdexcept>
 #include <string>
 
-#include "../kernels/wave_shuffle.h"
+#include "stack_device.h"
 #include "stack_ops.h"
 
 namespace omx {
 namespace stack {
-
-struct bf16 {
-  uint16_t v;
-};
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
-// round to nearest even, as torch's float -> bfloat16 conversion
-__device__ __forceinline__ uint16_t f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
-__device__ __forceinline__ float ld(const float* p) { return *p; }
-__device__ __forceinline__ float ld(const bf16* p) { return bf2f(p->v); }
-__device__ __forceinline__ void st(float* p, float v) { *p = v; }
-__device__ __forceinline__ void st(bf16* p, float v) { p->v = f2bf(v); }
-
-// butterfly reductions on DPP / permlane exchanges (wave_shuffle.h): no LDS round trip per dependent step
-__device__ __forceinline__ float wave_sum(float v) {
-  v += xor_shfl<32>(v);
-  v += xor_shfl<16>(v);
-  v += xor_shfl<8>(v);
-  v += xor_shfl<4>(v);
-  v += xor_shfl<2>(v);
-  v += xor_shfl<1>(v);
-  return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-  v = fmaxf(v, xor_shfl<32>(v));
-  v = fmaxf(v, xor_shfl<16>(v));
-  v = fmaxf(v, xor_shfl<8>(v));
-  v = fmaxf(v, xor_shfl<4>(v));
-  v = fmaxf(v, xor_shfl<2>(v));
-  v = fmaxf(v, xor_shfl<1>(v));
-  return v;
-}
-// sum over a block of 256 threads; every thread gets the result. red: 4 floats of LDS
-__device__ __forceinline__ float block_sum256(float v, float* red) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
-}
-__device__ __forceinline__ float silu(float z) { return z / (1.f + expf(-z)); }
-__device__ __forceinline__ float sigmoidf(float z) { return 1.f / (1.f + expf(-z)); }
-
-static void check(bool ok, const char* what) {
-  if (!ok) throw std::runtime_error(std::string("stack kernels: ") + what);
-}
-static void launched(const char* what) {
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) throw std::runtime_error(std::string("stack kernels: ") + what + ": " + hipGetErrorString(e));
-}
-
-// ------------------------------------------------------------------------------------------------
-// dot product of two rows over a wave: 16-byte loads when both rows allow it
-template <typename T>
-__device__ __forceinline__ float wave_dot(const T* __restrict__ w, const T* __restrict__ x, int K, int lane, bool vec);
-template <>
-__device__ __forceinline__ float wave_dot<bf16>(const bf16* __restrict__ w, const bf16* __restrict__ x, int K, int lane,
-                                                bool vec) {
-  float acc = 0.f;
-  if (vec) {
-    for (int k = lane * 8; k < K; k += 512) {
-      const u32x4 a = *(const u32x4*)(w + k), b = *(const u32x4*)(x + k);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc += __uint_as_float(a[i] << 16) * __uint_as_float(b[i] << 16);
-        acc += __uint_as_float(a[i] & 0xffff0000u) * __uint_as_float(b[i] & 0xffff0000u);
-      }
-    }
-  } else {
-    for (int k = lane; k < K; k += 64) acc += ld(w + k) * ld(x + k);
-  }
-  return wave_sum(acc);
-}
-template <>
-__device__ __forceinline__ float wave_dot<float>(const float* __restrict__ w, const float* __restrict__ x, int K, int lane,
-                                                 bool vec) {
-  float acc = 0.f;
-  if (vec) {
-    for (int k = lane * 4; k < K; k += 256) {
-      const f32x4 a = *(const f32x4*)(w + k), b = *(const f32x4*)(x + k);
-      acc += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
-    }
-  } else {
-    for (int k = lane; k < K; k += 64) acc += w[k] * x[k];
-  }
-  return wave_sum(acc);
-}
-template <typename T>
-static inline bool vec_ok(const void* p, long long ld_elems, int K) {
-  const int per = 16 / (int)sizeof(T);
-  return K % per == 0 && ld_elems % per == 0 && ((uintptr_t)p & 15) == 0;
-}
 
 // ------------------------------------------------------------------------------------------------ epilogue
 struct Epi {
@@ -530,22 +429,24 @@ void gemm(const GemmParams& P, hipStream_t s) {
 // ------------------------------------------------------------------------------------------------ embed / norm
 template <typename T>
 __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, int E,
-                                                    int V, float* __restrict__ resid, float* __restrict__ x0) {
+                                                    int V, float* __restrict__ resid, float* __restrict__ x0,
+                                                    float scale) {
   const int b = blockIdx.x;
   int t = tokens[b];
   t = t < 0 ? 0 : (t >= V ? V - 1 : t);
   for (int i = threadIdx.x; i < E; i += 256) {
-    const float v = ld(table + (long long)t * E + i);
+    const float v = ld(table + (long long)t * E + i) * scale;
     resid[(long long)b * E + i] = v;
     x0[(long long)b * E + i] = v;
   }
 }
-void embed(const void* table, const int* tokens, int B, int E, int V, float* resid, float* x0, int f32, hipStream_t s) {
+void embed(const void* table, const int* tokens, int B, int E, int V, float* resid, float* x0, float scale, int f32,
+           hipStream_t s) {
   check(B > 0 && table && tokens && resid && x0, "embed: bad operands");
   if (f32)
-    hipLaunchKernelGGL(embed_kernel<float>, dim3(B), dim3(256), 0, s, (const float*)table, tokens, E, V, resid, x0);
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(B), dim3(256), 0, s, (const float*)table, tokens, E, V, resid, x0, scale);
   else
-    hipLaunchKernelGGL(embed_kernel<bf16>, dim3(B), dim3(256), 0, s, (const bf16*)table, tokens, E, V, resid, x0);
+    hipLaunchKernelGGL(embed_kernel<bf16>, dim3(B), dim3(256), 0, s, (const bf16*)table, tokens, E, V, resid, x0, scale);
   launched("embed");
 }
 
@@ -683,6 +584,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
   const int* bt = R.block_table + (long long)R.q_seq[b] * R.max_blocks;
   const T* kc = (const T*)P.kc;
   const T* vc = (const T*)P.vc;
+  const long long ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;  // row strides of the pools
   float m[RQ], l[RQ], acc[RQ][DC];
 #pragma unroll
   for (int r = 0; r < RQ; ++r) {
@@ -704,12 +606,12 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
     float v0[UB][DC];
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-      const T* vr = vc + (long long)__builtin_amdgcn_readlane(rowidx, u) * P.Dv;  // a key past the end: row 0, weight 0
+      const T* vr = vc + (long long)__builtin_amdgcn_readlane(rowidx, u) * ldv;  // a key past the end: row 0, weight 0
 #pragma unroll
       for (int c = 0; c < DC; ++c) v0[u][c] = (lane + 64 * c < P.Dv) ? ld(vr + lane + 64 * c) : 0.f;
     }
     if (valid) {
-      const T* kr = kc + (long long)rowidx * P.D;
+      const T* kr = kc + (long long)rowidx * ldk;
       if (vec) {
         for (int d0 = 0; d0 < P.D; d0 += 64) {  // 64 dims of the row in flight at a time
           float k8[8][8];
@@ -765,7 +667,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
       float v[UB][DC];
 #pragma unroll
       for (int u = 0; u < UB; ++u) {
-        const T* vr = vc + (long long)__builtin_amdgcn_readlane(rowidx, j0 + u) * P.Dv;
+        const T* vr = vc + (long long)__builtin_amdgcn_readlane(rowidx, j0 + u) * ldv;
 #pragma unroll
         for (int c = 0; c < DC; ++c) v[u][c] = (lane + 64 * c < P.Dv) ? ld(vr + lane + 64 * c) : 0.f;
       }
@@ -805,12 +707,14 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
         for (int c = 0; c < DC; ++c) acc[r][c] += ag[w][r][lane + 64 * c] * f;
       }
       l[r] = L;
+      m[r] = M;
     }
   }
 #pragma unroll
   for (int r = 0; r < RQ; ++r) {
     if (r < nr) {
       T* out = (T*)P.out + (long long)b * P.ld_out + (h0 + r) * P.Dv;
+      if (P.sink) l[r] += expf(P.sink[h0 + r] - m[r]);  // the sink: a term of the denominator without key or value
       const float inv = 1.f / l[r];
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
@@ -841,6 +745,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
   const int* bt = R.block_table + (long long)R.q_seq[b] * R.max_blocks;
   const T* kc = (const T*)P.kc;
   const T* vc = (const T*)P.vc;
+  const long long ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
   const int kq = lane >> 4, dq = lane & 15;
   float m = -INFINITY, l = 0.f, acc[DPL];
 #pragma unroll
@@ -853,7 +758,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
     float dot = 0.f;
     if (valid) {
       rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
-      const T* kr = kc + (long long)rowidx * P.D;
+      const T* kr = kc + (long long)rowidx * ldk;
       if (vec) {
         for (int d0 = 0; d0 < P.D; d0 += 64) {
           float k8[8][8];
@@ -892,7 +797,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
     float v[16][DPL];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const T* vr = vc + (long long)rs[wv][kq * 16 + i] * P.Dv + dq * DPL;
+      const T* vr = vc + (long long)rs[wv][kq * 16 + i] * ldv + dq * DPL;
       if (vvec) {
         if (dq * DPL < P.Dv) {
           if constexpr (DPL == 4 && sizeof(T) == 2) {
@@ -963,6 +868,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
     return;
   }
   T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
+  if (P.sink) L += expf(P.sink[h] - M);
   const float inv = 1.f / L;
 #pragma unroll
   for (int c = 0; c < DPL; ++c)
@@ -982,6 +888,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnParams P, int 
     const float ms = w[(long long)sidx * (P.Dv + 2)];
     if (ms != -INFINITY) L += w[(long long)sidx * (P.Dv + 2) + 1] * expf(ms - M);  // a split without keys weighs nothing
   }
+  if (P.sink) L += expf(P.sink[item % P.H] - M);
   T* out = (T*)P.out + (long long)(item / P.H) * P.ld_out + (item % P.H) * P.Dv;
   for (int d = lane; d < P.Dv; d += 64) {
     float o = 0.f;
@@ -994,18 +901,19 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnParams P, int 
 }
 template <typename T>
 static void launch_attention_decode(const AttnParams& P, const StepRows& R, hipStream_t s) {
-  const int vec = P.D % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
+  const int ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
+  const int vec = P.D % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
   const int ns = (P.nsplit > 1 && P.split_ws && (long long)R.B * P.H * P.nsplit * (P.Dv + 2) <= P.split_ws_floats) ? P.nsplit : 1;
   dim3 grid(R.B * P.H, ns);
   const int per = 16 / (int)sizeof(T);  // elements of a 16-byte load
   if (P.Dv <= 64) {
-    const int vvec = P.Dv % 4 == 0 && (sizeof(T) == 2 ? 1 : 0) && ((uintptr_t)P.vc & 15) == 0;  // 8-byte pieces (bf16)
+    const int vvec = P.Dv % 4 == 0 && ldv % 4 == 0 && (sizeof(T) == 2 ? 1 : 0) && ((uintptr_t)P.vc & 15) == 0;  // 8-byte pieces (bf16)
     hipLaunchKernelGGL((attention_decode_kernel<T, 4>), grid, dim3(256), 0, s, P, R, vec, sizeof(T) == 2 ? vvec : 0, ns);
   } else if (P.Dv <= 128) {
-    const int vvec = P.Dv % 8 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
+    const int vvec = P.Dv % 8 == 0 && ldv % 8 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
     hipLaunchKernelGGL((attention_decode_kernel<T, 8>), grid, dim3(256), 0, s, P, R, vec, vvec, ns);
   } else {
-    const int vvec = P.Dv % 16 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
+    const int vvec = P.Dv % 16 == 0 && ldv % 8 == 0 && ((uintptr_t)P.vc & 15) == 0 && per <= 8;
     hipLaunchKernelGGL((attention_decode_kernel<T, 16>), grid, dim3(256), 0, s, P, R, vec, vvec, ns);
   }
   if (ns > 1)
@@ -1034,7 +942,7 @@ static void launch_attention(const AttnParams& P, const StepRows& R, hipStream_t
   const int per = P.H / P.G;
   const int rq = per >= 4 ? 4 : per >= 2 ? 2 : 1;
   const int nbatch = (per + rq - 1) / rq;
-  const int vec = P.D % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
+  const int vec = P.D % 8 == 0 && (P.ldk ? P.ldk : P.D) % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
   if (rq == 4)
     launch_attention_r<T, 4>(P, R, nbatch, vec, s);
   else if (rq == 2)
@@ -1220,7 +1128,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   }
 }
 bool flash_prefill_supported(const AttnParams& P) {
-  return !P.f32 && P.D == P.Dv && (P.D == 64 || P.D == 96 || P.D == 128) && P.ld % 4 == 0 && P.off_q % 4 == 0 &&
+  return !P.f32 && !P.sink && !P.ldk && !P.ldv && P.D == P.Dv && (P.D == 64 || P.D == 96 || P.D == 128) && P.ld % 4 == 0 && P.off_q % 4 == 0 &&
          ((uintptr_t)P.proj & 15) == 0 && ((uintptr_t)P.kc & 15) == 0 && ((uintptr_t)P.vc & 15) == 0;
 }
 void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s) {

@@ -34,7 +34,9 @@ void gemm(const GemmParams& P, hipStream_t s);
 int gemm_path(int M, int N, int K, int f32);
 void set_gemm_mfma(int on);  // 0: bfloat16 tiles also take the FMA kernel (A/B and tests)
 
-void embed(const void* table, const int* tokens, int B, int E, int V, float* resid, float* x0, int f32, hipStream_t s);
+// resid[r] = x0[r] = table[tokens[r]] * scale
+void embed(const void* table, const int* tokens, int B, int E, int V, float* resid, float* x0, float scale, int f32,
+           hipStream_t s);
 // out[r] = layer_norm(x[idx ? idx[r] : r]) * w + b, written in the matrix dtype
 void layer_norm_cast(const float* x, const int* idx, int rows, int E, const float* w, const float* b, float eps,
                      void* out, int f32, hipStream_t s);
@@ -67,6 +69,10 @@ struct AttnParams {
   int nsplit;
   float* split_ws;
   long long split_ws_floats;
+  // pools whose rows are wider than the head (0: D and Dv). With kc == vc and ldk == ldv the first Dv elements
+  // of a cached row are its value too (latent attention: one row per token serves every head)
+  int ldk, ldv;
+  const float* sink;    // [H] or null: exp(sink[h]) joins the softmax denominator (no key, no value, not scaled)
 };
 // q *= 1 + coef * ln(floor((pos + 1) / every) + 1); k, v of every row stored at its slot
 void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s);
@@ -137,8 +143,16 @@ struct MoeParams {
   int ld_hmid;
   float* y;             // [B][E] float32 feed-forward output
   int f32;
+  // score router (moe_route_scores): the last `identity` of the X + identity router outputs return their input;
+  // router_b is the choice correction; idw [B] receives the summed weight of the chosen identity outputs
+  int identity, group_count, group_keep;
+  float* idw;
 };
 void moe_route(const MoeParams& P, hipStream_t s);   // top-k ids + softmax weights, shared gate and activation
+// softmax over all router outputs, choice by score + correction inside the best expert groups, weights = the
+// chosen scores (not renormalised); leaves eids / ew / sgate (= 1) / the shared activation as moe_route does, so
+// moe_experts, moe_down and moe_grouped follow unchanged
+void moe_route_scores(const MoeParams& P, hipStream_t s);
 void moe_experts(const MoeParams& P, hipStream_t s); // gate/up + activation of the routed experts -> hmid
 void moe_down(const MoeParams& P, hipStream_t s);    // y = sum_j w_j down_j(hmid_j) + sgate * shared_down(hmid_s)
 // a few rows (decode steps): routing + routed and shared activations in one launch, then the experts' down
@@ -162,6 +176,79 @@ struct MoeGroupWs {
 };
 void moe_grouped(const MoeParams& P, const MoeGroupWs& W, hipStream_t s);
 bool moe_grouped_supported(const MoeParams& P);
+
+// ---- layers whose norm sits on the sublayer's output (stack_mixers.hip)
+// out = x in the matrix dtype (the sublayers read the stream itself)
+void cast_rows(const float* x, int rows, int E, void* out, int f32, hipStream_t s);
+// x[r] += layer_norm(y[r] + (idw ? idw[r] * x[r] : 0)) * w + b; hout (or null): the updated rows in the matrix dtype
+void post_norm_add(float* x, const float* y, int rows, int E, const float* w, const float* b, float eps, const float* idw,
+                   void* hout, int f32, hipStream_t s);
+
+struct LatentParams {
+  const float* proj;    // [B][ld] float32: per head [D plain | R rotated] queries at off_q, [C latent | R key part]
+  int ld, off_q, off_k, off_g;  // at off_k, the output gate's pre-activations [H * Dv] at off_g
+  int H, D, R, C, Dv;
+  int rot_dims;         // adjacent pairs (2i, 2i + 1), i < rot_dims / 2, of the rotated part turn
+  const double* inv_freq;  // [rot_dims / 2]
+  const float* norm_w;  // [C] weight of the latent's RMS norm
+  float eps;
+  const void* w_uk;     // [H * D][C]
+  const void* w_uvT;    // [H][C][Dv]
+  void* cache;          // [blocks][1][bs][C + R] matrix dtype
+  float* qa;            // [B][ld_qa]: per head [W_uk_h^T q_plain | rotated q part] (the attention's queries)
+  int ld_qa;
+  const void* lat;      // [B][ld_lat] matrix dtype: the attention's outputs in latent space, per head C
+  int ld_lat;
+  void* out;            // [B][ld_out] matrix dtype: (W_uv_h lat_h) * sigmoid(g), head-major
+  int ld_out;
+  int f32;
+};
+void latent_prepare(const LatentParams& P, const StepRows& R, hipStream_t s);
+void latent_expand(const LatentParams& P, int B, hipStream_t s);
+bool latent_supported(int D, int R, int C, int Dv);
+
+struct ConvParams {
+  const float* proj;    // [B][ld] float32: the convolution's inputs at off_in
+  int ld, off_in;
+  int ch, taps;
+  const float* w;       // [ch][taps], the last tap is the current token's
+  const float* bias;    // [ch]
+  float* state;         // slot s: state + s * state_stride = [taps - 1][ch], the sequence's last inputs
+  long long state_stride;
+  float* out;           // [B][ld_out] float32: silu(conv)
+  int ld_out;
+};
+void conv_silu(const ConvParams& P, const StepRows& R, hipStream_t s);
+
+enum { SCAN_MLSTM = 0, SCAN_SSD = 1 };
+struct ScanParams {
+  int mode;
+  const float* proj;    // [B][ld] float32
+  int ld;
+  const float* conv;    // SCAN_SSD: [B][ld_conv] the convolution's output (q, k, v live there)
+  int ld_conv;
+  int off_q, off_k, off_v;  // G groups of D (q, k), H heads of Dv (v)
+  int off_i, off_f;     // SCAN_MLSTM: gate pre-activations [H] in proj; SCAN_SSD: off_i = dt [H] in proj
+  int off_g;            // SCAN_SSD: z [H * Dv] in proj
+  int H, G, D, Dv;
+  const float* i_b;     // SCAN_MLSTM [H]
+  const float* f_b;
+  float cap;
+  const float* dt_bias; // SCAN_SSD [H]
+  const float* a_log;
+  const float* d_skip;
+  float* state;         // slot s: state + s * state_stride = S [H][D][Dv] (| n [H][D] | m [H] for SCAN_MLSTM)
+  long long state_stride;
+  float* y;             // [B][ld_y] float32
+  int ld_y;
+};
+void gated_scan(const ScanParams& P, const StepRows& R, hipStream_t s);
+bool gated_scan_supported(int mode, int D, int Dv);
+// out = y / rms(y over each of `groups` equal parts) * w * (gate ? sigmoid(gate) : 1), matrix dtype
+void group_rms_cast(const float* y, int ld_y, int rows, int n, int groups, const float* w, float eps, const float* gate,
+                    int ld_gate, void* out, int ld_out, int f32, hipStream_t s);
+// out = relu(z)^2, matrix dtype
+void relu2_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
 
 }  // namespace stack
 }  // namespace omx

@@ -24,7 +24,8 @@ import time
 
 import torch
 
-from ..models.config import MIX_ATTENTION, MIX_RETENTION
+from ..models.config import (BLOCK_POSTNORM, FF_DENSE, MIX_ATTENTION, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM,
+                             MIX_RETENTION)
 from .runner import Runner
 from .weights import StackWeights
 
@@ -40,10 +41,11 @@ class StackExec:
         self.r = r
         self.exe = e = C.Executor()
         w, cfg = r.w, r.cfg
+        self._f64 = []  # float64 rotary tables (kept alive here: the executor holds raw pointers)
         p = lambda t: t.data_ptr() if t is not None else 0  # noqa: E731
         e.configure(dict(E=cfg.n_embd, V=cfg.n_vocab, eps=float(cfg.norm_eps), residual_mult=float(cfg.residual_mult),
                          logit_softcap=float(cfg.logit_softcap), f32=int(w.dtype == torch.float32),
-                         max_B=r.max_batch, max_seqs=r.max_seqs))
+                         max_B=r.max_batch, max_seqs=r.max_seqs, block=int(cfg.block), embed_scale=float(cfg.embed_scale)))
         e.set_globals(dict(embed=p(w.embed), loop_in=p(w.loop_in), final_w=p(w.final_w), final_b=p(w.final_b),
                            head=p(w.head)))
         for i, (L, spec) in enumerate(zip(w.layers, cfg.layers)):
@@ -53,11 +55,25 @@ class StackExec:
                      n_in=L["n_in"], norm_w=p(L["norm_w"]), norm_b=p(L["norm_b"]), w_in=p(L["w_in"]), w_o=p(L["w_o"]),
                      decay=p(L.get("decay")), inv_freq=p(L.get("inv_freq")),
                      **{"off_" + k: v for k, v in L["off"].items()})
-            if f is not None:
+            if f is not None and f.kind == FF_DENSE:
+                d.update(ff=f.ff, ff_dense=1, w_dense_down=p(L["w_dense_down"]))
+            elif f is not None:
                 d.update(experts=f.experts, top=f.top, ff=f.ff, shared_ff=f.shared_ff, router_b=p(L["router_b"]),
-                         w_gu=p(L["w_gu"]), w_down=p(L["w_down"]), sh_down=p(L.get("sh_down")))
+                         w_gu=p(L["w_gu"]), w_down=p(L["w_down"]), sh_down=p(L.get("sh_down")), identity=f.identity,
+                         group_count=f.group_count, group_keep=f.group_keep)
+            if cfg.block == BLOCK_POSTNORM:  # norms on the sublayers' outputs: the feed-forward has its own input stack
+                if m.kind == MIX_LATENT and m.rot_dims:
+                    self._f64.append(L["inv_freq"].double().contiguous())
+                d.update(norm2_w=p(L.get("norm2_w")), norm2_b=p(L.get("norm2_b")), w_ff=p(L.get("w_ff")), n_ff=L["n_ff"],
+                         rot_dim=m.rot_dim, kv_rank=m.kv_rank, dkv_norm=p(L.get("dkv_norm")), w_uk=p(L.get("w_uk")),
+                         w_uvT=p(L.get("w_uvT")), sink=p(L.get("sink")), gate_cap=m.gate_cap, i_b=p(L.get("i_b")),
+                         f_b=p(L.get("f_b")), mnorm=p(L.get("mnorm")), state=m.state, groups=m.groups, conv=m.conv,
+                         norm_groups=m.norm_groups, conv_w=p(L.get("conv_w")), conv_b=p(L.get("conv_b")),
+                         dt_bias=p(L.get("dt_bias")), a_log=p(L.get("a_log")), d_skip=p(L.get("d_skip")),
+                         inv_freq64=p(self._f64[-1]) if m.kind == MIX_LATENT and m.rot_dims else 0, inv_freq=0)
             e.set_layer(i, d)
-        e.set_runs([dict(layer=li, opens_pass=int(first), kc=p(r.kc[ri]), vc=p(r.vc[ri]), state=p(r.states[ri]))
+        e.set_runs([dict(layer=li, opens_pass=int(first), kc=p(r.kc[ri]), vc=p(r.vc[ri]), state=p(r.states[ri]),
+                         state_stride=(r.states[ri].shape[1] if r.states[ri] is not None and r.states[ri].dim() == 2 else 0))
                     for ri, (li, _ps, first) in enumerate(r.runs)])
         e.set_workspace(dict(resid=p(r.resid), x0=p(r.x0), h=p(r.hbuf), cat=p(r.catbuf), proj=p(r.proj),
                              ld_proj=r.proj.shape[1], a=p(r.abuf), ld_a=r.abuf.shape[1], hmid=p(r.hmid),
@@ -65,7 +81,8 @@ class StackExec:
                              sgate=p(r.sgate), lrows=p(r.lbuf), obuf=p(r.obuf), ld_obuf=r.obuf.shape[1],
                              split_ws=p(r.split_ws), split_ws_floats=r.split_ws.numel(),
                              ret_chunks=p(r.d_chunks), ret_max_chunks=r.d_chunks.shape[0], ret_u=p(r.ret_u),
-                             ret_sin=p(r.ret_sin), ret_u_stride=r.ret_u.shape[1],
+                             ret_sin=p(r.ret_sin), ret_u_stride=r.ret_u.shape[1], cbuf=p(r.cbuf), ld_cbuf=r.cbuf.shape[1],
+                             lat=p(r.latbuf), ld_lat=r.latbuf.shape[1], idw=p(r.idw),
                              **{"moe_" + k: (v if isinstance(v, int) else p(v)) for k, v in r.moe_ws.items()}))
         e.set_inputs(dict(tokens=p(r.d_tokens), pos=p(r.d_pos), slot=p(r.d_slot), q_len=p(r.d_qlen),
                           q_seq=p(r.d_qseq), block_table=p(r.d_block_table), max_blocks=r.max_blocks,
@@ -150,19 +167,37 @@ class StackRunner(Runner):
                 self.kc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.dim, **tt))
                 self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
                 self.states.append(None)
-            else:
+            elif m.kind == MIX_LATENT:  # one row per token: latent | shared rotated key part (the latent is the value too)
+                self.kc.append(torch.zeros(n_blocks, 1, block_size, m.cache_dim, **tt))
+                self.vc.append(None)
+                self.states.append(None)
+            elif m.kind == MIX_RETENTION:
                 self.kc.append(None)
                 self.vc.append(None)
                 self.states.append(torch.zeros(max_seqs, m.heads, m.dim, m.vdim, **f32))
+            else:  # mLSTM: matrix memory | normaliser | running maximum; Mamba-2: state | the convolution's last inputs
+                self.kc.append(None)
+                self.vc.append(None)
+                self.states.append(torch.zeros(max_seqs, m.state_floats, **f32))
         mlps = [s.mlp for s in cfg.layers if s.mlp is not None]
-        top = max([f.top for f in mlps], default=1)
+        top = max([f.top for f in mlps] + [1])
         self.resid = torch.zeros(max_batch, E, **f32)
         self.x0 = torch.zeros(max_batch, E, **f32)          # the embedding output (re-enters at every pass)
         self.hbuf = torch.zeros(max_batch, E, **tt)         # normed activations, the input projection's operand
         self.catbuf = torch.zeros(max_batch, 2 * E, **tt)   # [x; x0], the pass-opening projection's operand
-        self.proj = torch.zeros(max_batch, (max(L["n_in"] for L in self.w.layers) + 3) // 4 * 4, **f32)  # rows 16-byte aligned
+        n_proj = max(max(L["n_in"], L.get("n_ff", 0)) for L in self.w.layers)
+        self.proj = torch.zeros(max_batch, (n_proj + 3) // 4 * 4, **f32)  # rows 16-byte aligned
         self.abuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **tt)
-        self.hmid = torch.zeros(max_batch, max([f.top * f.ff + f.shared_ff for f in mlps], default=1), **tt)
+        self.hmid = torch.zeros(max_batch, (max([f.ff if f.kind == FF_DENSE else f.top * f.ff + f.shared_ff for f in mlps],
+                                                default=1) + 7) // 8 * 8, **tt)
+        # latent attention: queries folded onto the latent (float32), outputs in latent space (matrix dtype);
+        # Mamba-2: the convolution's output (float32). idw: per-row weight of the chosen identity experts
+        lat = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_LATENT]
+        mam = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_MAMBA2]
+        self.cbuf = torch.zeros(max_batch, (max([m.heads * m.cache_dim for m in lat] + [m.conv_channels for m in mam],
+                                                default=1) + 3) // 4 * 4, **f32)
+        self.latbuf = torch.zeros(max_batch, (max([m.heads * m.kv_rank for m in lat], default=1) + 7) // 8 * 8, **tt)
+        self.idw = torch.zeros(max_batch, **f32)
         self.ybuf = torch.zeros(max_batch, E, **f32)
         self.eids = torch.zeros(max_batch, top, **i32)
         self.ew = torch.zeros(max_batch, top, **f32)

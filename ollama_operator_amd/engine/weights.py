@@ -414,7 +414,7 @@ class StackWeights:
     def __init__(self, path: str, device: str | torch.device = "cuda", dtype: torch.dtype = torch.bfloat16):
         import os as _os
 
-        from ..models.config import MIX_RETENTION, load_stack_config
+        from ..models.config import BLOCK_POSTNORM, MIX_RETENTION, load_stack_config
         from .safetensors_io import SafetensorsFile
         self.cfg = cfg = self.full_cfg = load_stack_config(path)
         self.device, self.dtype = device, dtype
@@ -434,10 +434,15 @@ class StackWeights:
         self.embed = mat(get("embed", (V, E)))
         self.loop_in = mat(get("loop.in", (E, 2 * E))) if cfg.loop_times else None
         self.layers = []
+        self._get, self._mat, self._vec = get, mat, vec
         for i, spec in enumerate(cfg.layers):
             m, f = spec.mixer, spec.mlp
             p = f"l{i}."
             L: dict = dict(norm_w=vec(get(p + "norm1", (E,))), norm_b=vec(get(p + "norm1.b", (E,))))
+            if cfg.block == BLOCK_POSTNORM:
+                self._load_postnorm_layer(L, p, spec)
+                self.layers.append(L)
+                continue
             parts = [get(p + "mix.q", (m.n_q, E)), get(p + "mix.k", (m.n_k, E)), get(p + "mix.v", (m.n_v, E))]
             off = dict(q=0, k=m.n_q, v=m.n_q + m.n_k)
             n = m.n_q + m.n_k + m.n_v
@@ -474,6 +479,68 @@ class StackWeights:
         self.final_w, self.final_b = vec(get("final.norm", (E,))), vec(get("final.norm.b", (E,)))
         self.head = mat(get("head", (V, E)))
         self.local = dict(E=E, V=V)
+
+    def _load_postnorm_layer(self, L: dict, p: str, spec) -> None:
+        """A layer whose sublayers read the stream itself and whose norms sit on their outputs. The mixer's
+        matrices that read the stream are one stacked `w_in`; the feed-forward reads the UPDATED stream, so its
+        input matrices (router | shared gate | shared up, or the dense up) are a second stack `w_ff`.
+        Latent attention keeps W_uk as stored ([H * dim][rank]: the query is folded onto the latent through it)
+        and W_uv transposed per head ([H][rank][vdim]: the latent-space output is expanded through it)."""
+        from ..models.config import FF_DENSE, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM
+        get, mat, vec = self._get, self._mat, self._vec
+        E, m, f, dev = self.cfg.n_embd, spec.mixer, spec.mlp, self.device
+        H, D, Dv = m.heads, m.dim, m.vdim
+        if m.kind == MIX_LATENT:
+            C, R = m.kv_rank, m.rot_dim
+            parts = [get(p + "mix.q", (H * (D + R), E)), get(p + "mix.dkv", (C + R, E)), get(p + "mix.g", (H * Dv, E))]
+            off = dict(q=0, k=H * (D + R), g=H * (D + R) + C + R)
+            L["dkv_norm"] = vec(get(p + "mix.dkv.norm", (C,)))
+            L["w_uk"] = mat(get(p + "mix.uk", (H * D, C)))
+            L["w_uvT"] = mat(get(p + "mix.uv", (H * Dv, C)).view(H, Dv, C).transpose(1, 2).reshape(H * C, Dv))
+            L["sink"] = vec(get(p + "mix.sink", (H,)))
+            L["inv_freq"] = (torch.from_numpy(rope_inv_freq(m.rot_dims, m.rot_base)).to(dev) if m.rot_dims else None)
+        elif m.kind == MIX_MLSTM:
+            parts = [get(p + "mix.q", (H * D, E)), get(p + "mix.k", (H * D, E)), get(p + "mix.v", (H * Dv, E)),
+                     get(p + "mix.g", (H * Dv, E)), get(p + "mix.i", (H, E)), get(p + "mix.f", (H, E))]
+            off = dict(q=0, k=H * D, v=2 * H * D, g=2 * H * D + H * Dv, i=2 * H * D + 2 * H * Dv, f=2 * H * D + 2 * H * Dv + H)
+            L["i_b"], L["f_b"] = vec(get(p + "mix.i.b", (H,))), vec(get(p + "mix.f.b", (H,)))
+            L["mnorm"] = vec(get(p + "mix.norm", (H * Dv,)))
+        elif m.kind == MIX_MAMBA2:
+            inner, GN, ch = H * Dv, m.groups * m.state, m.conv_channels
+            parts = [get(p + "mix.in", (2 * inner + 2 * GN + H, E))]
+            off = dict(g=0, conv=inner, dt=2 * inner + 2 * GN)      # z | x B C | dt
+            L["conv_w"], L["conv_b"] = vec(get(p + "mix.conv", (ch, m.conv))), vec(get(p + "mix.conv.b", (ch,)))
+            L["dt_bias"], L["a_log"], L["d_skip"] = (vec(get(p + "mix." + k, (H,))) for k in ("dt_bias", "A_log", "D"))
+            L["mnorm"] = vec(get(p + "mix.norm", (inner,)))
+        else:
+            raise ValueError("this block style has no mixer of that kind")
+        L["w_in"] = mat(*parts)
+        L["off"], L["n_in"] = off, sum(t.shape[0] for t in parts)
+        L["w_o"] = mat(get(p + "mix.o", (E, H * Dv)))
+        L["n_ff"] = 0
+        if f is None:
+            return
+        L["norm2_w"], L["norm2_b"] = vec(get(p + "norm2", (E,))), vec(get(p + "norm2.b", (E,)))
+        if f.kind == FF_DENSE:
+            L["w_ff"], L["n_ff"] = mat(get(p + "mlp.up", (f.ff, E))), f.ff
+            L["w_dense_down"] = mat(get(p + "mlp.down", (E, f.ff)))
+            return
+        X, F, Fs, NR = f.experts, f.ff, f.shared_ff, f.n_router
+        ff_parts = [get(p + "mlp.router", (NR, E))]
+        L["router_b"] = vec(get(p + "mlp.correction", (NR,)))
+        if Fs:
+            ff_parts += [get(p + "mlp.shared.gate", (Fs, E)), get(p + "mlp.shared.up", (Fs, E))]
+            off.update(sgate=NR, sup=NR + Fs)
+            L["sh_down"] = mat(get(p + "mlp.shared.down", (E, Fs)))
+        off["router"] = 0
+        L["w_ff"], L["n_ff"] = mat(*ff_parts), NR + 2 * Fs
+        gu, dn = [], []
+        for e in range(X):
+            q = f"{p}mlp.e{e}."
+            gu += [get(q + "gate", (F, E)), get(q + "up", (F, E))]
+            dn.append(get(q + "down", (E, F)))
+        L["w_gu"] = mat(*gu).view(X, 2 * F, E)
+        L["w_down"] = mat(*dn).view(X, E, F)
 
     @property
     def nbytes(self) -> int:

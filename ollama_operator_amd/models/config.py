@@ -246,6 +246,19 @@ def preset(name: str, **overrides) -> ModelConfig:
 
 MIX_ATTENTION = 0   # softmax attention over a paged key/value cache
 MIX_RETENTION = 1   # decayed linear attention with a per-sequence state matrix
+MIX_LATENT = 2      # softmax attention whose keys and values come from one cached low-rank latent per token
+MIX_MLSTM = 3       # matrix memory with exponential input / forget gates and a running stabiliser
+MIX_MAMBA2 = 4      # selective state space layer (scalar decay per head) behind a short causal convolution
+STATE_MIXERS = (MIX_RETENTION, MIX_MLSTM, MIX_MAMBA2)   # mixers that own a per-sequence state slot
+
+BLOCK_PARALLEL = 0  # x <- x + m (mixer(LN(x)) + ff(LN(x))): one norm, both sublayers read it
+BLOCK_POSTNORM = 1  # x <- x + LN1(mixer(x)), then x <- x + LN2(ff(x)): the norm sits on the sublayer's output
+
+FF_MOE = 0          # routed experts (+ shared expert)
+FF_DENSE = 1        # W_down act(W_up h), act = relu(z)^2
+ROUTE_TOPK_SOFTMAX = 0   # top-k of (logits + bias), softmax over the chosen logits
+ROUTE_SCORE_GROUPS = 1   # softmax over all outputs; choice by score + correction inside the best expert groups;
+                         # weights = the chosen scores; trailing outputs may be identity experts
 
 
 @dataclass
@@ -264,6 +277,18 @@ class MixerSpec:
     decay: tuple = ()           # per-head state decay
     rot_dims: int = 0           # rotary dims per head (rotate-half pairing), 0 = none
     rot_base: float = 10000.0
+    # latent attention: per head `dim` plain + `rot_dim` rotated query / key dims (adjacent-pair rotation of
+    # the first rot_dims of the rotated part), keys / values expanded from a latent of kv_rank; a per-head
+    # sink in the softmax denominator; sigmoid output gate
+    rot_dim: int = 0
+    kv_rank: int = 0
+    # mlstm
+    gate_cap: float = 0.0       # gate pre-activations pass cap * tanh(z / cap)
+    # mamba2: heads x vdim channels, `state` rows per head, `groups` shared B / C groups
+    state: int = 0
+    groups: int = 1
+    conv: int = 1               # taps of the causal convolution (the last one is the current token's)
+    norm_groups: int = 1        # the gated output is RMS-normed in this many equal parts
 
     @property
     def n_q(self) -> int:
@@ -281,6 +306,25 @@ class MixerSpec:
     def n_out(self) -> int:     # input width of the output projection
         return self.heads * self.vdim
 
+    @property
+    def conv_channels(self) -> int:   # mamba2: x | B | C pass the convolution
+        return self.heads * self.vdim + 2 * self.groups * self.state
+
+    @property
+    def cache_dim(self) -> int:       # latent attention: cached row = latent | shared rotated key part
+        return self.kv_rank + self.rot_dim
+
+    @property
+    def state_floats(self) -> int:
+        """float32 words of the per-sequence state of one run of this mixer."""
+        if self.kind == MIX_RETENTION:
+            return self.heads * self.dim * self.vdim
+        if self.kind == MIX_MLSTM:      # S [H][dim][vdim] | n [H][dim] | m [H]
+            return self.heads * (self.dim * self.vdim + self.dim + 1)
+        if self.kind == MIX_MAMBA2:     # S [H][state][vdim] | the convolution's last taps - 1 inputs
+            return self.heads * self.state * self.vdim + (self.conv - 1) * self.conv_channels
+        return 0
+
 
 @dataclass
 class MoESpec:
@@ -288,6 +332,16 @@ class MoESpec:
     top: int = 0
     ff: int = 0
     shared_ff: int = 0          # 0 = no shared expert
+    kind: int = FF_MOE          # FF_DENSE: only `ff` counts
+    route: int = ROUTE_TOPK_SOFTMAX
+    identity: int = 0           # trailing router outputs whose "expert" returns its input
+    group_count: int = 1        # experts (identity ones included) form this many groups of neighbours
+    group_keep: int = 1         # only experts of the best group_keep groups can be chosen
+    shared_gate: bool = True    # the shared expert sits behind a scalar sigmoid gate
+
+    @property
+    def n_router(self) -> int:
+        return self.experts + self.identity
 
 
 @dataclass
@@ -308,6 +362,8 @@ class StackConfig:
     norm_eps: float = 1e-5
     residual_mult: float = 1.0
     logit_softcap: float = 0.0
+    block: int = BLOCK_PARALLEL
+    embed_scale: float = 1.0
     ctx_len: int = 1 << 20      # the design has no positional table: bounded by the cache pool only
     bos_id: int = 0
     eos_id: int = -1            # no tokenizer ships with these models: generation never stops on a token
@@ -334,7 +390,7 @@ class StackConfig:
     @property
     def has_state(self) -> bool:
         """Some layer carries a recurrent state: a cached prefix cannot be cut back to an earlier length."""
-        return any(s.mixer.kind == MIX_RETENTION for s in self.layers)
+        return any(s.mixer.kind in STATE_MIXERS for s in self.layers)
 
     def to_dict(self) -> dict:
         return asdict(self)
@@ -415,8 +471,102 @@ class StackConfig:
             c["loop"] = dict(start=self.loop_start, stop=self.loop_stop, times=self.loop_times)
         return c
 
+    # -- config.json of the Norevik design
+    @classmethod
+    def from_norevik(cls, c: dict) -> "StackConfig":
+        def bad(msg):
+            raise UnsupportedArchitecture("Norevik: " + msg)
 
-STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix}
+        layers = []
+        for ent in c["layers"]:
+            m, t = ent["mixer"], ent["type"]
+            if t == "latent_attention":
+                rot = m.get("rot") or {}
+                mx = MixerSpec(kind=MIX_LATENT, heads=int(m["heads"]), kv_heads=1, dim=int(m["dim"]), vdim=int(m["vdim"]),
+                               scale=float(m["scale"]), rot_dim=int(m["rot_dim"]), kv_rank=int(m["kv_rank"]),
+                               rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)))
+                if mx.rot_dims % 2 or mx.rot_dims > mx.rot_dim:
+                    bad("rot.dims must be even and at most rot_dim")
+            elif t == "mlstm":
+                mx = MixerSpec(kind=MIX_MLSTM, heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]),
+                               vdim=int(m["vdim"]), gate_cap=float(m["gate_cap"]))
+                if mx.gate_cap <= 0:
+                    bad("gate_cap must be positive")
+            elif t == "mamba2":
+                mx = MixerSpec(kind=MIX_MAMBA2, heads=int(m["heads"]), kv_heads=int(m["groups"]), dim=int(m["state"]),
+                               vdim=int(m["vdim"]), state=int(m["state"]), groups=int(m["groups"]), conv=int(m["conv"]),
+                               norm_groups=int(m.get("norm_groups", 1)))
+                if mx.groups <= 0 or mx.heads % mx.groups:
+                    bad("heads must be a multiple of groups")
+                if mx.norm_groups <= 0 or (mx.heads * mx.vdim) % mx.norm_groups:
+                    bad("heads * vdim must be a multiple of norm_groups")
+                if mx.conv < 1:
+                    bad("conv must be at least 1")
+            else:
+                raise UnsupportedArchitecture(f"unknown mixer type {t!r}")
+            if min(mx.heads, mx.dim, mx.vdim) <= 0:
+                bad("mixer sizes must be positive")
+            mlp = None
+            f = ent.get("mlp")
+            if f:
+                kind = f.get("kind")
+                if kind == "dense":
+                    mlp = MoESpec(kind=FF_DENSE, ff=int(f["ff"]))
+                elif kind == "moe":
+                    r, sh = f["router"], f.get("shared") or {}
+                    gr = r.get("groups") or {}
+                    mlp = MoESpec(kind=FF_MOE, route=ROUTE_SCORE_GROUPS, experts=int(r["experts"]), top=int(r["top"]),
+                                  ff=int(f["expert"]["ff"]), shared_ff=int(sh.get("ff", 0)), identity=int(r.get("identity", 0)),
+                                  group_count=int(gr.get("count", 1)), group_keep=int(gr.get("keep", gr.get("count", 1))),
+                                  shared_gate=False)
+                    if not 0 < mlp.top <= mlp.n_router:
+                        bad("router: top must be in 1..experts + identity")
+                    if mlp.group_count < 1 or mlp.n_router % mlp.group_count or not 0 < mlp.group_keep <= mlp.group_count:
+                        bad("router: groups must divide the router outputs, keep in 1..count")
+                    if mlp.group_keep * (mlp.n_router // mlp.group_count) < mlp.top:
+                        bad("router: the kept groups hold fewer experts than top")
+                else:
+                    raise UnsupportedArchitecture(f"unknown feed-forward kind {kind!r}")
+            layers.append(LayerSpec(mixer=mx, mlp=mlp))
+        return cls(arch="norevik", n_vocab=int(c["vocab"]), n_embd=int(c["width"]), layers=layers,
+                   norm_eps=float(c["norm"]["eps"]), block=BLOCK_POSTNORM,
+                   embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)), name=str(c.get("name", "")))
+
+    def to_norevik(self) -> dict:
+        """The config.json this configuration is read from (random-init fixtures, tests)."""
+        out = []
+        for s in self.layers:
+            m = s.mixer
+            if m.kind == MIX_LATENT:
+                ent = dict(type="latent_attention", mixer=dict(
+                    heads=m.heads, dim=m.dim, rot_dim=m.rot_dim, vdim=m.vdim, kv_rank=m.kv_rank, scale=m.scale,
+                    rot=dict(dims=m.rot_dims, base=m.rot_base)))
+            elif m.kind == MIX_MLSTM:
+                ent = dict(type="mlstm", mixer=dict(heads=m.heads, dim=m.dim, vdim=m.vdim, gate_cap=m.gate_cap))
+            elif m.kind == MIX_MAMBA2:
+                ent = dict(type="mamba2", mixer=dict(heads=m.heads, vdim=m.vdim, state=m.state, groups=m.groups,
+                                                      conv=m.conv, norm_groups=m.norm_groups))
+            else:
+                raise UnsupportedArchitecture("Norevik has no mixer of this kind")
+            f = s.mlp
+            if f is None:
+                ent["mlp"] = None
+            elif f.kind == FF_DENSE:
+                ent["mlp"] = dict(kind="dense", ff=f.ff)
+            else:
+                ent["mlp"] = dict(kind="moe", expert=dict(ff=f.ff),
+                                  router=dict(experts=f.experts, top=f.top, identity=f.identity,
+                                              groups=dict(count=f.group_count, keep=f.group_keep)),
+                                  **({"shared": dict(ff=f.shared_ff)} if f.shared_ff else {}))
+            out.append(ent)
+        return dict(architecture="Norevik", vocab=self.n_vocab, width=self.n_embd, layers=out,
+                    norm=dict(eps=self.norm_eps), embedding=dict(scale=self.embed_scale))
+
+    def to_config_json(self) -> dict:
+        return self.to_norevik() if self.arch == "norevik" else self.to_bizulix()
+
+
+STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix, "Norevik": StackConfig.from_norevik}
 
 
 def is_stack_model(path: str) -> bool:

@@ -256,20 +256,148 @@ def stack_route(z: torch.Tensor, top: int):
     return idx.to(torch.int32), torch.softmax(val, -1)
 
 
+# ---- layers whose norm sits on the sublayer's output (BLOCK_POSTNORM): latent attention, mLSTM, Mamba-2,
+# dense and score-routed feed-forwards. One function per kernel of csrc/stack/stack_mixers.hip.
+
+def stack_post_norm_add(x, y, w, b, eps, idw=None):
+    """x += layer_norm(y + idw * x) * w + b (idw: per-row weight of the identity experts, or None)."""
+    if idw is not None:
+        y = y + idw[:, None] * x
+    x += F.layer_norm(y, (y.shape[-1],), w, b, eps)
+
+
+def stack_rotate_pairs(x, pos, inv_freq):
+    """x [B, ..., R] float32: dims (2i, 2i + 1), i < len(inv_freq), turn by pos * inv_freq[i] (float64 angles)."""
+    n = inv_freq.numel()
+    ang = pos.double()[:, None] * inv_freq.double()[None, :]
+    while ang.dim() < x.dim():
+        ang = ang.unsqueeze(1)
+    c, s = torch.cos(ang).float(), torch.sin(ang).float()
+    u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    out = x.clone()
+    out[..., 0:2 * n:2] = u * c - v * s
+    out[..., 1:2 * n:2] = v * c + u * s
+    return out
+
+
+def stack_latent_prepare(proj, off, m, L, pos, slot, cache, bs, eps):
+    """The cached row of every token, [rms_norm(latent) * w | rotated shared key part], stored at its slot; returns
+    the queries folded onto the latent: per head [W_uk_h^T q_plain | rotated q part], float32 [B, H, C + R]."""
+    B, H, D, R, C = proj.shape[0], m.heads, m.dim, m.rot_dim, m.kv_rank
+    q = proj[:, off["q"]:off["q"] + H * (D + R)].view(B, H, D + R)
+    dkv = proj[:, off["k"]:off["k"] + C + R]
+    c = dkv[:, :C] * torch.rsqrt(dkv[:, :C].pow(2).mean(-1, keepdim=True) + eps) * L["dkv_norm"]
+    kr, qr = dkv[:, C:], q[..., D:]
+    if L["inv_freq"] is not None:
+        kr, qr = stack_rotate_pairs(kr, pos, L["inv_freq"]), stack_rotate_pairs(qr, pos, L["inv_freq"])
+    blk, o = slot.long() // bs, slot.long() % bs
+    cache[blk, 0, o] = torch.cat([c, kr], 1).to(cache.dtype)
+    qa = torch.einsum("bhd,hdc->bhc", q[..., :D], L["w_uk"].float().view(H, D, C))
+    return torch.cat([qa, qr], -1)
+
+
+def stack_latent_attention(qa, cache, C, block_table, q_seq, q_len, bs, scale, sink):
+    """qa [B, H, C + R]; cache [blocks, 1, bs, C + R]; the first C dims of a cached row are also its value.
+    softmax with exp(sink_h) added to the denominator. Returns float32 [B, H, C]."""
+    B, H, _ = qa.shape
+    out = torch.empty(B, H, C, dtype=torch.float32, device=qa.device)
+    for b in range(B):
+        n = int(q_len[b])
+        t = torch.arange(n, device=qa.device)
+        bt = block_table[int(q_seq[b])].long()
+        kk = cache[bt[t // bs], 0, t % bs].float()            # [n, C + R]
+        s = (qa[b] @ kk.T) * scale                            # [H, n]
+        mx = torch.maximum(s.max(-1, keepdim=True).values, sink[:, None])
+        e = torch.exp(s - mx)
+        out[b] = (e / (e.sum(-1, keepdim=True) + torch.exp(sink[:, None] - mx))) @ kk[:, :C]
+    return out
+
+
+def stack_conv_silu(xin, w, bias, state, q_seq):
+    """Causal per-channel convolution over each sequence's rows, continued from `state` [slots, taps - 1, ch]
+    (the sequence's last inputs, oldest first), which is advanced in place. xin [B, ch] -> silu(conv) [B, ch]."""
+    B, K = xin.shape[0], w.shape[1]
+    out = torch.empty_like(xin)
+    for b in range(B):
+        st = state[int(q_seq[b])]
+        win = torch.cat([st, xin[b:b + 1]], 0)                 # [K, ch], last row = the current token
+        out[b] = F.silu((win * w.T).sum(0) + bias)
+        if K > 1:
+            st.copy_(win[1:])
+    return out
+
+
+def stack_gated_scan(q, k, v, a, b, S, q_seq, kv_group=1):
+    """S [slots, H, D, Dv] <- a S + b k v^T per row (a, b [B, H]), o = S^T q. q, k [B, G, D] with head h using
+    group h // kv_group; v [B, H, Dv]. Returns float32 [B, H, Dv]."""
+    B, H = a.shape
+    out = torch.empty_like(v)
+    hg = torch.arange(H, device=v.device) // kv_group
+    for r in range(B):
+        St = S[int(q_seq[r])]
+        St.mul_(a[r][:, None, None]).add_((b[r][:, None] * k[r][hg])[:, :, None] * v[r][:, None, :])
+        out[r] = torch.einsum("hdv,hd->hv", St, q[r][hg])
+    return out
+
+
+def stack_mlstm_gates(i_raw, f_raw, cap, m_state, q_seq):
+    """Per row and head: decay a = exp(f + m' - m), input weight b = exp(i - m) with m = max(f + m', i), m' the
+    running maximum of the sequence (m_state [slots, H], advanced in place). Returns a, b, m [B, H]."""
+    ig = cap * torch.tanh(i_raw / cap)
+    fg = F.logsigmoid(cap * torch.tanh(f_raw / cap))
+    a, b, mm = torch.empty_like(ig), torch.empty_like(ig), torch.empty_like(ig)
+    for r in range(ig.shape[0]):
+        mp = m_state[int(q_seq[r])]
+        mn = torch.maximum(fg[r] + mp, ig[r])
+        a[r], b[r], mm[r] = torch.exp(fg[r] + mp - mn), torch.exp(ig[r] - mn), mn
+        mp.copy_(mn)
+    return a, b, mm
+
+
+def stack_group_rms(y, groups, w, eps, gate=None):
+    """y [B, n] in `groups` equal parts, each divided by its root mean square; times w; times sigmoid(gate)."""
+    B, n = y.shape
+    g = y.view(B, groups, n // groups)
+    o = (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)).reshape(B, n) * w
+    return o * torch.sigmoid(gate) if gate is not None else o
+
+
+def stack_route_scores(z, corr, top, n_real, group_count, group_keep):
+    """Router logits [B, X + I] -> softmax scores; the `top` largest of score + correction within the best
+    `group_keep` of `group_count` neighbour groups (a group's rank: its largest corrected score). Returns expert
+    ids [B, top] (identity choices point at expert 0 with weight 0), weights [B, top] and the summed weight of
+    the chosen identity outputs [B]."""
+    s = torch.softmax(z, -1)
+    choice = s + corr
+    if group_count > 1:
+        per = z.shape[1] // group_count
+        best = choice.view(-1, group_count, per).max(-1).values
+        keep = torch.topk(best, group_keep, dim=-1).indices
+        ok = torch.zeros_like(best, dtype=torch.bool).scatter_(1, keep, True)
+        choice = choice.masked_fill(~ok.repeat_interleave(per, dim=1), -float("inf"))
+    ids = torch.topk(choice, top, dim=-1).indices
+    wt = torch.gather(s, 1, ids)
+    ident = ids >= n_real
+    idw = (wt * ident).sum(-1)
+    return torch.where(ident, 0, ids).to(torch.int32), torch.where(ident, 0.0, wt), idw
+
+
 class TorchStackExecutor:
     def __init__(self, runner):
         self.r = runner
 
     def embed(self, B: int):
         r = self.r
-        x = r.w.embed[r.d_tokens[:B].long()].float()
+        x = r.w.embed[r.d_tokens[:B].long()].float() * float(getattr(r.cfg, "embed_scale", 1.0))
         r.resid[:B] = x
         r.x0[:B] = x
 
     def layer_run(self, ri: int, B: int):
-        from ..models.config import MIX_ATTENTION
+        from ..models.config import BLOCK_POSTNORM, MIX_ATTENTION
         r = self.r
         w, cfg, T = r.w, r.cfg, r.w.dtype
+        if cfg.block == BLOCK_POSTNORM:
+            return self.layer_run_postnorm(ri, B)
         li, _ps, opens = r.runs[ri]
         L, spec = w.layers[li], cfg.layers[li]
         m, f, off = spec.mixer, spec.mlp, L["off"]
@@ -322,6 +450,89 @@ class TorchStackExecutor:
                 ff += torch.sigmoid(proj[:, off["sg"]:off["sg"] + 1]) * stack_matmul(mid, L["sh_down"])
             y = y + ff
         r.resid[:B] = x + cfg.residual_mult * y
+
+    def layer_run_postnorm(self, ri: int, B: int):
+        """x <- x + LN1(mixer(x)), then x <- x + LN2(ff(x)); both sublayers read the stream itself."""
+        from ..models.config import FF_DENSE, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM
+        r = self.r
+        w, cfg, T = r.w, r.cfg, r.w.dtype
+        li = r.runs[ri][0]
+        L, spec = w.layers[li], cfg.layers[li]
+        m, f, off = spec.mixer, spec.mlp, L["off"]
+        H, D, Dv, n_out = m.heads, m.dim, m.vdim, m.n_out
+        x = r.resid[:B]
+        pos, qseq = r.d_pos[:B], r.d_qseq[:B]
+        r.hbuf[:B] = x.to(T)
+        proj = stack_matmul(r.hbuf[:B], L["w_in"])
+        r.proj[:B, :proj.shape[1]] = proj
+        if m.kind == MIX_LATENT:
+            C = m.kv_rank
+            qa = stack_latent_prepare(proj, off, m, L, pos, r.d_slot[:B], r.kc[ri], r.block_size, cfg.norm_eps)
+            lat = stack_latent_attention(qa, r.kc[ri], C, r.d_block_table, qseq, r.d_qlen[:B], r.block_size, m.scale,
+                                         L["sink"])
+            r.latbuf[:B, :H * C] = lat.reshape(B, H * C).to(T)
+            o = torch.einsum("bhc,hcv->bhv", r.latbuf[:B, :H * C].float().view(B, H, C), L["w_uvT"].float().view(H, C, Dv))
+            a = o.reshape(B, n_out) * torch.sigmoid(proj[:, off["g"]:off["g"] + n_out])
+        elif m.kind == MIX_MLSTM:
+            st = r.states[ri]
+            nS = H * D * Dv
+            S, nv, ms = st[:, :nS].view(-1, H, D, Dv), st[:, nS:nS + H * D].view(-1, H, D, 1), st[:, nS + H * D:]
+            q = proj[:, off["q"]:off["q"] + H * D].view(B, H, D) * float(D) ** -0.5
+            k = proj[:, off["k"]:off["k"] + H * D].view(B, H, D)
+            v = proj[:, off["v"]:off["v"] + n_out].view(B, H, Dv)
+            ga, gb, mm = stack_mlstm_gates(proj[:, off["i"]:off["i"] + H] + L["i_b"], proj[:, off["f"]:off["f"] + H] + L["f_b"],
+                                           m.gate_cap, ms, qseq)
+            o = stack_gated_scan(q, k, v, ga, gb, S, qseq)
+            nq = stack_gated_scan(q, k, torch.ones(B, H, 1), ga, gb, nv, qseq)
+            o = o / (torch.maximum(nq.abs(), torch.exp(-mm)[..., None]) + 1e-6)
+            a = stack_group_rms(o.reshape(B, n_out), H, L["mnorm"], cfg.norm_eps, proj[:, off["g"]:off["g"] + n_out])
+        else:
+            assert m.kind == MIX_MAMBA2
+            st = r.states[ri]
+            N, G, ch = m.state, m.groups, m.conv_channels
+            nS = H * N * Dv
+            S, cst = st[:, :nS].view(-1, H, N, Dv), st[:, nS:].view(-1, m.conv - 1, ch)
+            xbc = stack_conv_silu(proj[:, off["conv"]:off["conv"] + ch], L["conv_w"].view(ch, m.conv), L["conv_b"], cst, qseq)
+            xs = xbc[:, :n_out].view(B, H, Dv)
+            Bm = xbc[:, n_out:n_out + G * N].view(B, G, N)
+            Cm = xbc[:, n_out + G * N:].view(B, G, N)
+            dt = F.softplus(proj[:, off["dt"]:off["dt"] + H] + L["dt_bias"])
+            ga = torch.exp(-torch.exp(L["a_log"]) * dt)
+            y = stack_gated_scan(Cm, Bm, xs, ga, dt, S, qseq, kv_group=H // G) + L["d_skip"][None, :, None] * xs
+            y = y.reshape(B, n_out) * F.silu(proj[:, off["g"]:off["g"] + n_out])
+            a = stack_group_rms(y, m.norm_groups, L["mnorm"], cfg.norm_eps)
+        r.abuf[:B, :n_out] = a.to(T)
+        r.ybuf[:B] = stack_matmul(r.abuf[:B, :n_out], L["w_o"])
+        stack_post_norm_add(x, r.ybuf[:B], L["norm_w"], L["norm_b"], cfg.norm_eps)
+        if f is None:
+            return
+        r.hbuf[:B] = x.to(T)
+        h = r.hbuf[:B]
+        proj = stack_matmul(h, L["w_ff"])
+        r.proj[:B, :proj.shape[1]] = proj
+        idw = None
+        if f.kind == FF_DENSE:
+            r.hmid[:B, :f.ff] = torch.relu(proj).pow(2).to(T)
+            y = stack_matmul(r.hmid[:B, :f.ff], L["w_dense_down"])
+        else:
+            ids, wt, idw = stack_route_scores(proj[:, :f.n_router], L["router_b"], f.top, f.experts, f.group_count,
+                                              f.group_keep)
+            r.eids[:B, :f.top], r.ew[:B, :f.top] = ids, wt
+            y = torch.zeros_like(x)
+            for b in range(B):
+                for j in range(f.top):
+                    if float(wt[b, j]) == 0.0:
+                        continue
+                    e = int(ids[b, j])
+                    gu = stack_matmul(h[b:b + 1], L["w_gu"][e])[0]
+                    mid = (F.silu(gu[:f.ff]) * gu[f.ff:]).to(T)
+                    y[b] += wt[b, j] * stack_matmul(mid[None], L["w_down"][e])[0]
+            if f.shared_ff:
+                Fs = f.shared_ff
+                mid = (F.silu(proj[:, off["sgate"]:off["sgate"] + Fs]) * proj[:, off["sup"]:off["sup"] + Fs]).to(T)
+                y += stack_matmul(mid, L["sh_down"])
+        r.ybuf[:B] = y
+        stack_post_norm_add(x, r.ybuf[:B], L["norm2_w"], L["norm2_b"], cfg.norm_eps, idw)
 
     def head(self, n_logits: int, use_idx: bool):
         r = self.r
