@@ -212,7 +212,8 @@ class StackRunner(Runner):
         self.ret_u = torch.zeros(n_ch, max([m.heads * m.dim * m.vdim for m in rets], default=1) if n_ch > 1 else 1, **f32)
         self.ret_sin = torch.zeros_like(self.ret_u)
         # decode attention over long contexts: partials {maximum, sum, output} of up to 16 splits per (row, head)
-        hv = max([s.mixer.heads * (s.mixer.vdim + 2) for s in cfg.layers if s.mixer.kind == MIX_ATTENTION], default=1)
+        hv = max([s.mixer.heads * (s.mixer.vdim + 2) for s in cfg.layers if s.mixer.kind == MIX_ATTENTION] +
+                 [s.mixer.heads * (s.mixer.kv_rank + 2) for s in cfg.layers if s.mixer.kind == MIX_LATENT], default=1)
         self.split_ws = torch.zeros(16 * 16 * hv, **f32)
         self._step_rows = None  # (positions, sequence rows) of the rows last uploaded, until a step consumes them
         # routed feed-forward of prompt portions (bfloat16): pairs sorted by expert, per-expert matrix-core products

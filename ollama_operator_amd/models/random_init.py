@@ -64,6 +64,8 @@ def write_random_stack(path: str, cfg, seed: int = 0, std: float = 0.05) -> None
 
     from ..engine.safetensors_io import write_safetensors
     from .config import MIX_RETENTION
+    if cfg.arch == "norevik":
+        return write_random_norevik(path, cfg, seed=seed)
     g = torch.Generator().manual_seed(seed)
     E, V = cfg.n_embd, cfg.n_vocab
     T: dict = {}
@@ -101,5 +103,93 @@ def write_random_stack(path: str, cfg, seed: int = 0, std: float = 0.05) -> None
     rnd("head", (V, E), 1.0 / E ** 0.5)
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as fh:
-        json.dump(cfg.to_bizulix(), fh, indent=1)
+        json.dump(cfg.to_config_json(), fh, indent=1)
+    write_safetensors(os.path.join(path, "model.safetensors"), T)
+
+
+def write_random_norevik(path: str, cfg, seed: int = 0) -> None:
+    """Random-init model folder of the Norevik design (its tensor names). Projections ~ N(0, 1 / fan-in); norm
+    weights near 1; forget-gate biases positive (memories that last), step-size biases negative, decays spread
+    over several orders, sinks of a few units, router corrections of the size of a score."""
+    import json
+    import os
+
+    import torch
+
+    from ..engine.safetensors_io import write_safetensors
+    from .config import FF_DENSE, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM
+    g = torch.Generator().manual_seed(seed)
+    E, V = cfg.n_embd, cfg.n_vocab
+    T: dict = {}
+
+    def rnd(name, shape, s, mean=0.0):
+        T[name] = (mean + s * torch.randn(*shape, generator=g)).to(torch.bfloat16)
+
+    def uni(name, shape, lo, hi):
+        T[name] = (lo + (hi - lo) * torch.rand(*shape, generator=g)).to(torch.bfloat16)
+
+    def lin(name, n_out, n_in, gain=1.0):
+        rnd(name, (n_out, n_in), gain / n_in ** 0.5)
+
+    def norm(name, n):
+        rnd(name, (n,), 0.1, 1.0)
+        rnd(name + ".b", (n,), 0.1)
+
+    rnd("embed", (V, E), 1.0 / max(cfg.embed_scale, 1e-6))
+    for i, spec in enumerate(cfg.layers):
+        m, f, p = spec.mixer, spec.mlp, f"l{i}."
+        H, D, Dv = m.heads, m.dim, m.vdim
+        norm(p + "norm1", E)
+        if m.kind == MIX_LATENT:
+            lin(p + "mix.q", H * (D + m.rot_dim), E, 2.0)
+            lin(p + "mix.dkv", m.kv_rank + m.rot_dim, E, 2.0)
+            rnd(p + "mix.dkv.norm", (m.kv_rank,), 0.1, 1.0)
+            lin(p + "mix.uk", H * D, m.kv_rank, 1.5)
+            lin(p + "mix.uv", H * Dv, m.kv_rank)
+            uni(p + "mix.sink", (H,), -1.0, 4.0)
+            lin(p + "mix.g", H * Dv, E, 1.5)
+        elif m.kind == MIX_MLSTM:
+            lin(p + "mix.q", H * D, E)
+            lin(p + "mix.k", H * D, E)
+            lin(p + "mix.v", H * Dv, E)
+            lin(p + "mix.g", H * Dv, E, 1.5)
+            lin(p + "mix.i", H, E, 2.0)
+            lin(p + "mix.f", H, E, 2.0)
+            rnd(p + "mix.i.b", (H,), 1.0)
+            uni(p + "mix.f.b", (H,), 0.5, 6.0)
+            rnd(p + "mix.norm", (H * Dv,), 0.1, 1.0)
+        elif m.kind == MIX_MAMBA2:
+            inner, ch = H * Dv, m.conv_channels
+            lin(p + "mix.in", 2 * inner + 2 * m.groups * m.state + H, E)
+            rnd(p + "mix.conv", (ch, m.conv), 0.6, 0.2)
+            rnd(p + "mix.conv.b", (ch,), 0.1)
+            uni(p + "mix.dt_bias", (H,), -4.0, -0.5)
+            uni(p + "mix.A_log", (H,), -4.0, 1.0)
+            uni(p + "mix.D", (H,), 0.5, 1.0)
+            rnd(p + "mix.norm", (inner,), 0.1, 1.0)
+        else:
+            raise ValueError("the Norevik design has no mixer of this kind")
+        lin(p + "mix.o", E, H * Dv)
+        if f is None:
+            continue
+        norm(p + "norm2", E)
+        if f.kind == FF_DENSE:
+            lin(p + "mlp.up", f.ff, E)
+            lin(p + "mlp.down", E, f.ff)
+            continue
+        for e in range(f.experts):
+            lin(f"{p}mlp.e{e}.gate", f.ff, E)
+            lin(f"{p}mlp.e{e}.up", f.ff, E)
+            lin(f"{p}mlp.e{e}.down", E, f.ff)
+        lin(p + "mlp.router", f.n_router, E, 3.0)
+        rnd(p + "mlp.correction", (f.n_router,), 0.3)
+        if f.shared_ff:
+            lin(p + "mlp.shared.gate", f.shared_ff, E)
+            lin(p + "mlp.shared.up", f.shared_ff, E)
+            lin(p + "mlp.shared.down", E, f.shared_ff)
+    norm("final.norm", E)
+    lin("head", V, E)
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as fh:
+        json.dump(cfg.to_norevik(), fh, indent=1)
     write_safetensors(os.path.join(path, "model.safetensors"), T)

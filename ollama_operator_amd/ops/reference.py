@@ -491,7 +491,7 @@ class TorchStackExecutor:
             st = r.states[ri]
             N, G, ch = m.state, m.groups, m.conv_channels
             nS = H * N * Dv
-            S, cst = st[:, :nS].view(-1, H, N, Dv), st[:, nS:].view(-1, m.conv - 1, ch)
+            S, cst = st[:, :nS].view(-1, H, N, Dv), st[:, nS:].view(st.shape[0], m.conv - 1, ch)
             xbc = stack_conv_silu(proj[:, off["conv"]:off["conv"] + ch], L["conv_w"].view(ch, m.conv), L["conv_b"], cst, qseq)
             xs = xbc[:, :n_out].view(B, H, Dv)
             Bm = xbc[:, n_out:n_out + G * N].view(B, G, N)
