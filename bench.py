@@ -357,6 +357,39 @@ STACK_SIZES = {
 }
 
 
+# the Norevik design at the same widths: latent attention x2, an mLSTM and a Mamba-2 layer, twice; the first layer's
+# feed-forward is dense, the others route 2 of 8 experts + 2 identity outputs in 2 groups, beside a shared expert
+NOREVIK_SIZES = {
+    "s": dict(E=1024, pattern="llxm" * 2, H=16, D=64, R=32, Dv=64, C=192, F=512, X=8, top=2, Fs=1024, dense=2048,
+              mlstm=(8, 64, 128), mamba=(16, 64, 64, 1)),
+    "m": dict(E=2048, pattern="llxm" * 2, H=16, D=128, R=64, Dv=128, C=192, F=1024, X=8, top=2, Fs=2048, dense=4096,
+              mlstm=(16, 64, 128), mamba=(32, 64, 128, 2)),
+}
+
+
+def norevik_config(z: dict, vocab: int = 32000):
+    """A Norevik model with the sizes of a real model's layers (random weights)."""
+    from ollama_operator_amd.models.config import (BLOCK_POSTNORM, FF_DENSE, FF_MOE, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM,
+                                                    ROUTE_SCORE_GROUPS, LayerSpec, MixerSpec, MoESpec, StackConfig)
+    layers = []
+    for i, c in enumerate(z["pattern"]):
+        if c == "l":
+            m = MixerSpec(kind=MIX_LATENT, heads=z["H"], kv_heads=1, dim=z["D"], vdim=z["Dv"], rot_dim=z["R"], kv_rank=z["C"],
+                          scale=(z["D"] + z["R"]) ** -0.5, rot_dims=z["R"], rot_base=1e4)
+        elif c == "x":
+            h, d, dv = z["mlstm"]
+            m = MixerSpec(kind=MIX_MLSTM, heads=h, kv_heads=h, dim=d, vdim=dv, gate_cap=15.0)
+        else:
+            h, dv, n, g = z["mamba"]
+            m = MixerSpec(kind=MIX_MAMBA2, heads=h, kv_heads=g, dim=n, vdim=dv, state=n, groups=g, conv=4, norm_groups=g)
+        f = (MoESpec(kind=FF_DENSE, ff=z["dense"]) if i == 0 else
+             MoESpec(kind=FF_MOE, route=ROUTE_SCORE_GROUPS, experts=z["X"], top=z["top"], ff=z["F"], shared_ff=z["Fs"],
+                     identity=2, group_count=2, group_keep=1, shared_gate=False))
+        layers.append(LayerSpec(mixer=m, mlp=f))
+    return StackConfig(arch="norevik", n_vocab=vocab, n_embd=z["E"], layers=layers, norm_eps=1e-5, block=BLOCK_POSTNORM,
+                       embed_scale=float(z["E"]) ** 0.5)
+
+
 def stack_config(z: dict, vocab: int = 32000):
     """A Bizulix model with the sizes of a real model's layers (random weights)."""
     from ollama_operator_amd.models.config import (MIX_ATTENTION, MIX_RETENTION, LayerSpec, MixerSpec, MoESpec,
@@ -424,6 +457,15 @@ def bench_stack(a) -> None:
         r.warmup()
         out[name] = {"bizulix_bf16": measure(r), "weights_gb": round(r.w.nbytes / 1e9, 3)}
         r.close()
+        if a.norevik:  # the Norevik design at the same width and depth, through the same engine and measurement
+            d = os.path.join(a.dir, f"norevik-{name}")
+            if not os.path.exists(os.path.join(d, "model.safetensors")):
+                write_random_stack(d, norevik_config(NOREVIK_SIZES[name]), seed=0)
+            r = StackRunner(d, device="cuda:0", dtype="bfloat16", max_batch=a.chunk, max_seqs=2, ctx=ctx)
+            r.warmup()
+            out[name]["norevik_bf16"] = measure(r)
+            out[name]["norevik_weights_gb"] = round(r.w.nbytes / 1e9, 3)
+            r.close()
         if not a.stack_only:
             cfg = ModelConfig(name=f"mixtral-like-{name}", n_vocab=32000, n_embd=z["E"], n_layer=len(z["pattern"]),
                               n_head=z["H"], n_head_kv=z["G"], n_ff=z["F"], n_rot=z["D"], n_embd_head=z["D"],
@@ -446,6 +488,8 @@ def main():
                     "Bizulix design at these sizes beside the closest GGUF model at equal size, instead of the "
                     "default workload")
     ap.add_argument("--stack-only", action="store_true", help="with --stack: skip the comparison model")
+    ap.add_argument("--norevik", action="store_true", help="with --stack: also measure the Norevik design (latent "
+                    "attention, mLSTM, Mamba-2, score-routed experts) at the same widths")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--tp", type=int, default=1, help="tensor-parallel degree: one sequence sharded over T GPUs")
     ap.add_argument("--allow-shared", action="store_true",

@@ -50,6 +50,7 @@ PYBIND11_MODULE(_stack, m) {
   m.def("retention_supported", &retention_supported);
   m.def("gated_scan_supported", &gated_scan_supported);
   m.def("latent_supported", &latent_supported);
+  m.def("gated_chunk_rows", &gated_chunk_rows);
   m.def("retention_chunk_rows", &retention_chunk_rows);
   m.attr("FLASH_TILE_ROWS") = (int)FLASH_TILE_ROWS;
 
@@ -127,6 +128,8 @@ PYBIND11_MODULE(_stack, m) {
         L.dkv_norm = Pp<const float>(ptr(d, "dkv_norm"));
         L.w_uk = Pp<const void>(ptr(d, "w_uk"));
         L.w_uvT = Pp<const void>(ptr(d, "w_uvT"));
+        L.w_ukT = Pp<const void>(ptr(d, "w_ukT"));
+        L.w_uv = Pp<const void>(ptr(d, "w_uv"));
         L.sink = Pp<const float>(ptr(d, "sink"));
         L.gate_cap = getf(d, "gate_cap");
         L.off_i = geti(d, "off_i");
@@ -202,6 +205,9 @@ PYBIND11_MODULE(_stack, m) {
         w.lat = Pp<void>(ptr(d, "lat"));
         w.ld_lat = geti(d, "ld_lat");
         w.idw = Pp<float>(ptr(d, "idw"));
+        w.coef = Pp<float>(ptr(d, "coef"));
+        w.ld_coef = geti(d, "ld_coef");
+        w.ctot = Pp<float>(ptr(d, "ctot"));
       })
       .def("set_inputs", [](StackExecutor& e, py::dict d) {
         StackInputs& in = e.in;

@@ -79,6 +79,16 @@ void StackExecutor::embed(int B, hipStream_t s) {
   stack::embed(embed_w, in.tokens, B, cfg.E, cfg.V, ws.resid, ws.x0, cfg.embed_scale, cfg.f32, s);
 }
 
+static ScanChunkWs scan_ws(const StackExecutor& e) {
+  return ScanChunkWs{e.ws.ret.chunks, e.n_chunks, e.ws.ret.max_chunks, e.ws.ret.U, e.ws.ret.Sin, e.ws.ret.u_stride, e.ws.coef,
+                     e.ws.ctot, e.ws.ret.obuf, e.ws.ret.ld_o};
+}
+static bool chunked_scan_ok(const StackExecutor& e, const ScanParams& P, int B) {
+  const int dvp = P.Dv + (P.mode == SCAN_MLSTM ? 1 : 0);
+  return B > SMALL_B && e.n_chunks > 0 && e.ws.ret.U && e.ws.ret.Sin && e.ws.coef && e.ws.ctot && e.ws.ld_coef >= 3 * P.H &&
+         e.ws.ret.u_stride >= (long long)P.H * P.D * dvp && e.ws.ret.ld_o >= P.H * dvp && gated_chunk_supported(P.mode, P.D, P.Dv);
+}
+
 // x <- x + LN1(mixer(x)), then x <- x + LN2(ff(x)): both sublayers read the stream itself (cast to the matrix
 // dtype), the layer norm sits on their outputs.
 void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
@@ -94,7 +104,7 @@ void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
   if (L.kind == 2) {
     const int C = L.kv_rank, W = C + L.rot_dim;
     LatentParams P{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_g, L.heads, L.dim, L.rot_dim, C, L.vdim, L.rot_dims,
-                   L.inv_freq64, L.dkv_norm, cfg.eps, L.w_uk, L.w_uvT, r.kc, ws.cbuf, ws.ld_cbuf, ws.lat, ws.ld_lat, ws.a,
+                   L.inv_freq64, L.dkv_norm, cfg.eps, L.w_uk, L.w_uvT, L.w_ukT, L.w_uv, r.kc, ws.cbuf, ws.ld_cbuf, ws.lat, ws.ld_lat, ws.a,
                    ws.ld_a, f32};
     latent_prepare(P, R, s);
     // one cached row per token serves every head: attention with a single key/value head whose key is the whole
@@ -121,11 +131,17 @@ void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
     P.cap = L.gate_cap;
     P.state = r.state;
     P.state_stride = r.state_stride;
+    P.off_g = L.off_g;
     P.y = ws.ret.obuf;
     P.ld_y = ws.ret.ld_o;
-    gated_scan(P, R, s);
-    // per-head unit RMS, the norm's weight, the sigmoid output gate
-    group_rms_cast(ws.ret.obuf, ws.ret.ld_o, B, n_out, L.heads, L.mnorm, cfg.eps, ws.proj + L.off_g, ws.ld_proj, ws.a, ws.ld_a, f32, s);
+    if (chunked_scan_ok(*this, P, B)) {  // prompt portions: chunks in parallel around a scan over the chunk states
+      gated_scan_chunked(P, R, scan_ws(*this), L.mnorm, cfg.eps, ws.a, ws.ld_a, f32, s);
+    } else {
+      gated_scan(P, R, s);
+      // per-head unit RMS, the norm's weight, the sigmoid output gate
+      group_rms_cast(ws.ret.obuf, ws.ret.ld_o, B, n_out, L.heads, L.mnorm, cfg.eps, ws.proj + L.off_g, ws.ld_proj, ws.a, ws.ld_a,
+                     f32, s);
+    }
   } else {
     const int ch = n_out + 2 * L.groups * L.state;
     ConvParams Cv{ws.proj, ws.ld_proj, L.off_conv, ch, L.conv, L.conv_w, L.conv_b,
@@ -153,7 +169,10 @@ void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
     P.state_stride = r.state_stride;
     P.y = ws.ret.obuf;
     P.ld_y = ws.ret.ld_o;
-    gated_scan(P, R, s);
+    if (chunked_scan_ok(*this, P, B))
+      gated_scan_chunked(P, R, scan_ws(*this), nullptr, cfg.eps, nullptr, 0, f32, s);
+    else
+      gated_scan(P, R, s);
     group_rms_cast(ws.ret.obuf, ws.ret.ld_o, B, n_out, L.norm_groups, L.mnorm, cfg.eps, nullptr, 0, ws.a, ws.ld_a, f32, s);
   }
   {

@@ -51,6 +51,8 @@ struct LayerDesc {
   const float* dkv_norm = nullptr;
   const void* w_uk = nullptr;
   const void* w_uvT = nullptr;
+  const void* w_ukT = nullptr;
+  const void* w_uv = nullptr;
   const float* sink = nullptr;
   float gate_cap = 0.f;             // mLSTM
   int off_i = 0, off_f = 0;
@@ -99,6 +101,9 @@ struct StackWorkspace {
   void* lat = nullptr;     // [max_B][ld_lat] matrix dtype: attention outputs in latent space
   int ld_lat = 0;
   float* idw = nullptr;    // [max_B] weight of the chosen identity experts
+  float* coef = nullptr;   // [max_B][ld_coef] chunked gated scan: per (row, head) {ln a, b, m}
+  int ld_coef = 0;
+  float* ctot = nullptr;   // [max chunks][ld_coef / 3] the chunks' summed ln a per head
   MoeGroupWs moe{};        // grouped routed feed-forward (prompt portions, bfloat16); gu == null: unused
   RetChunkWs ret{};        // chunked retention (prompt portions): chunk table, per-chunk states, o before its norm
 };

@@ -131,10 +131,13 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(LatentParams P, Ste
     P.qa[(long long)b * P.ld_qa + h * W + C + j] = rotate_pair_elem(qr, j, P.rot_dims, R.pos[b], P.inv_freq);
   }
 }
-// out[b][h * Dv + j] = (sum_c W_uvT[h][c][j] lat[b][h * C + c]) * sigmoid(g[b][h * Dv + j]); grid (row groups, H)
+// out[b][h * Dv + j] = (sum_c W_uvT[h][c][j] lat[b][h * C + c]) * sigmoid(g[b][h * Dv + j]); grid (row groups, H,
+// tiles of 64 columns). Thread (cg, jj) = (tid / 64, tid % 64) sums a quarter of the latent axis for column jj of the
+// tile (W_uvT is read along its contiguous axis); the four quarters meet in LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_expand_kernel(LatentParams P, int B) {
   __shared__ float ls[LAT_RB][LAT_MAXC];
+  __shared__ float part[4][LAT_RB][64];
   const int r0 = blockIdx.x * LAT_RB, h = blockIdx.y, tid = threadIdx.x;
   const int nr = min(LAT_RB, B - r0);
   const int C = P.C, Dv = P.Dv;
@@ -142,23 +145,111 @@ __global__ __launch_bounds__(256) void latent_expand_kernel(LatentParams P, int 
     const int i = idx / C, c = idx % C;
     ls[i][c] = ld((const T*)P.lat + (long long)(r0 + i) * P.ld_lat + h * C + c);
   }
+  for (int idx = tid; idx < (LAT_RB - nr) * C; idx += 256) ls[nr + idx / C][idx % C] = 0.f;
   __syncthreads();
+  const int cg = tid >> 6, jj = tid & 63, j = blockIdx.z * 64 + jj;
+  const int per = (C + 3) / 4, c0 = cg * per, c1 = min(C, c0 + per);
   const T* wv = (const T*)P.w_uvT + (long long)h * C * Dv;
-  for (int j = tid; j < Dv; j += 256) {
-    float acc[LAT_RB];
+  float acc[LAT_RB];
 #pragma unroll
-    for (int i = 0; i < LAT_RB; ++i) acc[i] = 0.f;
-    for (int c = 0; c < C; ++c) {
+  for (int i = 0; i < LAT_RB; ++i) acc[i] = 0.f;
+  if (j < Dv) {
+#pragma unroll 8
+    for (int c = c0; c < c1; ++c) {
       const float w = ld(wv + (long long)c * Dv + j);
 #pragma unroll
       for (int i = 0; i < LAT_RB; ++i) acc[i] += ls[i][c] * w;
     }
+  }
 #pragma unroll
-    for (int i = 0; i < LAT_RB; ++i)
-      if (i < nr) {
-        const float g = P.proj[(long long)(r0 + i) * P.ld + P.off_g + h * Dv + j];
-        st((T*)P.out + (long long)(r0 + i) * P.ld_out + h * Dv + j, acc[i] * sigmoidf(g));
+  for (int i = 0; i < LAT_RB; ++i) part[cg][i][jj] = acc[i];
+  __syncthreads();
+  for (int idx = tid; idx < nr * 64; idx += 256) {
+    const int i = idx >> 6, col = blockIdx.z * 64 + (idx & 63);
+    if (col < Dv) {
+      const float o = part[0][i][idx & 63] + part[1][i][idx & 63] + part[2][i][idx & 63] + part[3][i][idx & 63];
+      const float g = P.proj[(long long)(r0 + i) * P.ld + P.off_g + h * Dv + col];
+      st((T*)P.out + (long long)(r0 + i) * P.ld_out + h * Dv + col, o * sigmoidf(g));
+    }
+  }
+}
+// ---- decode steps (a few rows): the fold and the expansion as wave-per-output-row products, so every weight row is
+// one 16-byte load per lane and all of them are in flight at once (the row-group kernels above walk a weight column
+// with dependent 2-byte loads: fine when 8 rows share them from cache, slow when one row streams them from memory).
+// They read the other layouts of the two matrices: W_uk transposed per head [H][C][D], W_uv as stored [H * Dv][C].
+template <typename T>
+__device__ __forceinline__ float wave_dot_f32x(const T* __restrict__ w, const float* __restrict__ x, int K, int lane, bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int k = lane * 8; k < K; k += 512) {
+      float w8[8];
+      if constexpr (sizeof(T) == 2) {
+        const u32x4 a = *(const u32x4*)(w + k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          w8[2 * i] = __uint_as_float(a[i] << 16);
+          w8[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u);
+        }
+      } else {
+        const f32x4 a = *(const f32x4*)(w + k), b = *(const f32x4*)(w + k + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          w8[i] = a[i];
+          w8[4 + i] = b[i];
+        }
       }
+      const f32x4 xa = *(const f32x4*)(x + k), xb = *(const f32x4*)(x + k + 4);
+      acc += w8[0] * xa[0] + w8[1] * xa[1] + w8[2] * xa[2] + w8[3] * xa[3] + w8[4] * xb[0] + w8[5] * xb[1] + w8[6] * xb[2] +
+             w8[7] * xb[3];
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) acc += ld(w + k) * x[k];
+  }
+  return wave_sum(acc);
+}
+// blocks [0, nfold): wave (h, c) -> qa[b][h * W + c] = W_ukT[h][c][:] . q_plain_h(b) for every row b;
+// blocks nfold + b: row b's cache entry and the rotated parts of its queries
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prepare_small_kernel(LatentParams P, StepRows R, int nfold, int vec) {
+  __shared__ float red[4];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int C = P.C, Rr = P.R, D = P.D, W = C + Rr;
+  if ((int)blockIdx.x < nfold) {
+    const int item = blockIdx.x * 4 + (tid >> 6);
+    if (item >= P.H * C) return;
+    const int h = item / C, c = item % C;
+    const T* w = (const T*)P.w_ukT + (long long)item * D;
+    for (int b = 0; b < R.B; ++b) {
+      const float v = wave_dot_f32x<T>(w, P.proj + (long long)b * P.ld + P.off_q + h * (D + Rr), D, lane, vec != 0);
+      if (lane == 0) P.qa[(long long)b * P.ld_qa + h * W + c] = v;
+    }
+    return;
+  }
+  const int b = blockIdx.x - nfold;
+  const float* dkv = P.proj + (long long)b * P.ld + P.off_k;
+  float sq = 0.f;
+  for (int c = tid; c < C; c += 256) sq += dkv[c] * dkv[c];
+  const float inv = 1.f / sqrtf(block_sum256(sq, red) / (float)C + P.eps);
+  T* dst = (T*)P.cache + (long long)R.slot[b] * W;
+  for (int c = tid; c < C; c += 256) st(dst + c, dkv[c] * inv * P.norm_w[c]);
+  for (int j = tid; j < Rr; j += 256) st(dst + C + j, rotate_pair_elem(dkv + C, j, P.rot_dims, R.pos[b], P.inv_freq));
+  for (int idx = tid; idx < P.H * Rr; idx += 256) {
+    const int h = idx / Rr, j = idx % Rr;
+    const float* qr = P.proj + (long long)b * P.ld + P.off_q + h * (D + Rr) + D;
+    P.qa[(long long)b * P.ld_qa + h * W + C + j] = rotate_pair_elem(qr, j, P.rot_dims, R.pos[b], P.inv_freq);
+  }
+}
+// wave (h, j) -> out[b][h * Dv + j] = (W_uv[h * Dv + j][:] . lat[b][h * C :]) * sigmoid(g[b][h * Dv + j]) for every row b
+template <typename T>
+__global__ __launch_bounds__(256) void latent_expand_small_kernel(LatentParams P, int B, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= P.H * P.Dv) return;
+  const int h = item / P.Dv;
+  const T* w = (const T*)P.w_uv + (long long)item * P.C;
+  for (int b = 0; b < B; ++b) {
+    const float v = wave_dot<T>(w, (const T*)P.lat + (long long)b * P.ld_lat + h * P.C, P.C, lane, vec != 0);
+    if (lane == 0) st((T*)P.out + (long long)b * P.ld_out + item, v * sigmoidf(P.proj[(long long)b * P.ld + P.off_g + item]));
   }
 }
 bool latent_supported(int D, int R, int C, int Dv) {
@@ -169,8 +260,21 @@ static void check_latent(const LatentParams& P) {
             latent_supported(P.D, P.R, P.C, P.Dv) && P.rot_dims % 2 == 0 && P.rot_dims <= P.R && (P.rot_dims == 0 || P.inv_freq),
         "latent attention: operands or sizes (dim <= 256, kv_rank <= 512, kv_rank + rot_dim <= 256)");
 }
+constexpr int LAT_SMALL = 8;  // steps of at most this many rows take the wave-per-output kernels
 void latent_prepare(const LatentParams& P, const StepRows& R, hipStream_t s) {
   check_latent(P);
+  if (R.B <= LAT_SMALL && P.w_ukT) {
+    const int nfold = (P.H * P.C + 3) / 4;
+    const int per = P.f32 ? 4 : 8;
+    const int vec = P.D % 8 == 0 && (P.D + P.R) % 4 == 0 && P.off_q % 4 == 0 && P.ld % 4 == 0 && ((uintptr_t)P.proj & 15) == 0 &&
+                    ((uintptr_t)P.w_ukT & 15) == 0 && P.D % per == 0;
+    if (P.f32)
+      hipLaunchKernelGGL(latent_prepare_small_kernel<float>, dim3(nfold + R.B), dim3(256), 0, s, P, R, nfold, vec);
+    else
+      hipLaunchKernelGGL(latent_prepare_small_kernel<bf16>, dim3(nfold + R.B), dim3(256), 0, s, P, R, nfold, vec);
+    launched("latent_prepare_small");
+    return;
+  }
   const dim3 grid((R.B + LAT_RB - 1) / LAT_RB, P.H + 1);
   if (P.f32)
     hipLaunchKernelGGL(latent_prepare_kernel<float>, grid, dim3(256), 0, s, P, R);
@@ -180,7 +284,19 @@ void latent_prepare(const LatentParams& P, const StepRows& R, hipStream_t s) {
 }
 void latent_expand(const LatentParams& P, int B, hipStream_t s) {
   check_latent(P);
-  const dim3 grid((B + LAT_RB - 1) / LAT_RB, P.H);
+  if (B <= LAT_SMALL && P.w_uv) {
+    const dim3 grid((P.H * P.Dv + 3) / 4);
+    if (P.f32) {
+      const int vec = vec_ok<float>(P.w_uv, P.C, P.C) && vec_ok<float>(P.lat, P.ld_lat, P.C);
+      hipLaunchKernelGGL(latent_expand_small_kernel<float>, grid, dim3(256), 0, s, P, B, vec);
+    } else {
+      const int vec = vec_ok<bf16>(P.w_uv, P.C, P.C) && vec_ok<bf16>(P.lat, P.ld_lat, P.C);
+      hipLaunchKernelGGL(latent_expand_small_kernel<bf16>, grid, dim3(256), 0, s, P, B, vec);
+    }
+    launched("latent_expand_small");
+    return;
+  }
+  const dim3 grid((B + LAT_RB - 1) / LAT_RB, P.H, (P.Dv + 63) / 64);
   if (P.f32)
     hipLaunchKernelGGL(latent_expand_kernel<float>, grid, dim3(256), 0, s, P, B);
   else
@@ -191,21 +307,26 @@ void latent_expand(const LatentParams& P, int B, hipStream_t s) {
 // ------------------------------------------------------------------------------------------------ short convolution
 // out[r][c] = silu(bias[c] + sum_j w[c][j] in(p_r - (taps - 1) + j)[c]): tap taps - 1 is the current token's.
 // Inputs before the step's first row of the sequence come from its carried window (the last taps - 1 inputs,
-// oldest first; zero for a new sequence). One block per row. A second launch advances the windows: the block of
-// a sequence's LAST row of the step writes them (ascending, so a thread never reads what it has overwritten).
+// oldest first; zero for a new sequence). One block per row. A sequence with a single row in the step advances its
+// window there and then; for the others a second launch does: the block of a sequence's LAST row of the step writes
+// the window (ascending, so a thread never reads what it has overwritten).
 __global__ __launch_bounds__(256) void conv_silu_kernel(ConvParams P, StepRows R) {
   const int r = blockIdx.x, K = P.taps;
   const int seq = R.q_seq[r];
   int nb = 0;  // rows of the same sequence right before r, up to taps - 1
   while (nb < K - 1 && r - nb - 1 >= 0 && R.q_seq[r - nb - 1] == seq) ++nb;
-  const float* win = P.state + (long long)seq * P.state_stride;
+  // a sequence with ONE row in this step (a decode step): nobody else reads its window, so this block advances it
+  const bool alone = nb == 0 && !(r + 1 < R.B && R.q_seq[r + 1] == seq);
+  float* win = P.state + (long long)seq * P.state_stride;
   for (int c = threadIdx.x; c < P.ch; c += 256) {
     float acc = P.bias[c];
+    const float cur = P.proj[(long long)r * P.ld + P.off_in + c];
     for (int j = 0; j < K; ++j) {
       const int back = K - 1 - j;
-      const float v = back <= nb ? P.proj[(long long)(r - back) * P.ld + P.off_in + c]
-                                 : win[(long long)(K - 1 - (back - nb)) * P.ch + c];
+      const float v = back == 0 ? cur : back <= nb ? P.proj[(long long)(r - back) * P.ld + P.off_in + c]
+                                                   : win[(long long)(K - 1 - (back - nb)) * P.ch + c];
       acc += P.w[(long long)c * K + j] * v;
+      if (alone && back > 0) win[(long long)(K - 1 - back) * P.ch + c] = back == 1 ? cur : win[(long long)(K - back) * P.ch + c];
     }
     P.out[(long long)r * P.ld_out + c] = silu(acc);
   }
@@ -214,6 +335,7 @@ __global__ __launch_bounds__(256) void conv_window_kernel(ConvParams P, StepRows
   const int r = blockIdx.x, K = P.taps;
   const int seq = R.q_seq[r];
   if (r + 1 < R.B && R.q_seq[r + 1] == seq) return;  // not the sequence's last row of this step
+  if (!(r > 0 && R.q_seq[r - 1] == seq)) return;     // its only row: the first launch advanced the window
   int n = 1;  // rows of the sequence in this step, up to taps - 1
   while (n < K - 1 && r - n >= 0 && R.q_seq[r - n] == seq) ++n;
   float* win = P.state + (long long)seq * P.state_stride;
@@ -229,7 +351,7 @@ void conv_silu(const ConvParams& P, const StepRows& R, hipStream_t s) {
         "conv_silu: bad operands");
   hipLaunchKernelGGL(conv_silu_kernel, dim3(R.B), dim3(256), 0, s, P, R);
   launched("conv_silu");
-  if (P.taps > 1) {
+  if (P.taps > 1 && R.B > 1) {  // a single row is alone in its sequence
     hipLaunchKernelGGL(conv_window_kernel, dim3(R.B), dim3(256), 0, s, P, R);
     launched("conv_window");
   }
@@ -239,26 +361,25 @@ void conv_silu(const ConvParams& P, const StepRows& R, hipStream_t s) {
 // S_t = a_t S_(t-1) + b_t k_t v_t^T (S is D x Dv per head), o_t = S_t^T q_t, with per-row scalars
 //   SCAN_MLSTM: i = cap tanh((i_raw + i_b) / cap), f = logsigmoid(cap tanh((f_raw + f_b) / cap)),
 //               m_t = max(f + m_(t-1), i), a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); q scaled by D^(-1/2); a
-//               normaliser n_t = a n_(t-1) + b k_t rides along as one more column of S (v = 1), and
+//               normaliser n_t = a n_(t-1) + b k_t rides along, and
 //               y = o / (max(|n_t . q|, exp(-m_t)) + 1e-6)
 //   SCAN_SSD:   dt = softplus(dt_raw + dt_bias), a = exp(-exp(A_log) dt), b = dt; q = C_t, k = B_t of the head's
 //               group, v = x_t (all three from the convolution's output); y = (o + D x_t) silu(z_t)
 // One block per (sequence segment of the step, head), as the retention kernel: the block of the segment's first
-// row walks its rows; thread (g, j) = (tid / Dvp, tid % Dvp) keeps S[i][j], i = g, g + NG, ..., in registers
-// (Dvp = Dv columns + the normaliser's), so the update needs no exchange and o is a sum of NG partials per column.
-// The slot's state (S, then for the mLSTM n and m) is read once and written back once per step.
+// row walks its rows; thread (g, j) = (tid / Dv, tid % Dv) keeps S[i][j], i = g, g + NG, ..., in registers, so the
+// update needs no exchange and o is a sum of NG partials per column; the mLSTM's normaliser sits with threads
+// tid < D. The slot's state (S, then for the mLSTM n and m) is read once and written back once per step.
 __device__ __forceinline__ float softplusf(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 __device__ __forceinline__ float logsigmoidf(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 template <int MODE, int MAXI>
 __global__ __launch_bounds__(256) void gated_scan_kernel(ScanParams P, StepRows R) {
-  __shared__ float qs[256], ks[256], vs[260], po[256], os[260];
+  __shared__ float qs[256], ks[256], vs[256], po[256], os[256], nred[4];
   const int r0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int seq = R.q_seq[r0];
   if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;  // not the first row of its segment (uniform per block)
   const int D = P.D, Dv = P.Dv;
-  const int Dvp = Dv + (MODE == SCAN_MLSTM ? 1 : 0);
-  const int NG = 256 / Dvp;
-  const int g = tid / Dvp, j = tid % Dvp;
+  const int NG = 256 / Dv;
+  const int g = tid / Dv, j = tid % Dv;
   const bool act = g < NG;
   const int hg = h / (P.H / P.G);
   float* sbase = P.state + (long long)seq * P.state_stride;
@@ -269,19 +390,15 @@ __global__ __launch_bounds__(256) void gated_scan_kernel(ScanParams P, StepRows 
 #pragma unroll
   for (int ii = 0; ii < MAXI; ++ii) {
     const int i = g + ii * NG;
-    S[ii] = (act && i < D) ? (j < Dv ? S0[(long long)i * Dv + j] : nvec[i]) : 0.f;
+    S[ii] = (act && i < D) ? S0[(long long)i * Dv + j] : 0.f;
   }
+  // the mLSTM's normaliser n [D] lives with threads tid < D; its product with q is a sum over the block's waves
+  float nreg = (MODE == SCAN_MLSTM && tid < D) ? nvec[tid] : 0.f;
   float m = MODE == SCAN_MLSTM ? *mptr : 0.f;
   const float qscale = MODE == SCAN_MLSTM ? 1.f / sqrtf((float)D) : 1.f;
   for (int r = r0; r < R.B && R.q_seq[r] == seq; ++r) {
     const float* row = P.proj + (long long)r * P.ld;
     const float* src = MODE == SCAN_MLSTM ? row : P.conv + (long long)r * P.ld_conv;
-    if (tid < D) {
-      qs[tid] = src[P.off_q + hg * D + tid] * qscale;
-      ks[tid] = src[P.off_k + hg * D + tid];
-    }
-    if (tid < Dv) vs[tid] = src[P.off_v + h * Dv + tid];
-    if (MODE == SCAN_MLSTM && tid == Dv) vs[Dv] = 1.f;
     float a, b;
     if (MODE == SCAN_MLSTM) {
       const float ig = P.cap * tanhf((row[P.off_i + h] + P.i_b[h]) / P.cap);
@@ -294,6 +411,19 @@ __global__ __launch_bounds__(256) void gated_scan_kernel(ScanParams P, StepRows 
       const float dt = softplusf(row[P.off_i + h] + P.dt_bias[h]);
       a = expf(-expf(P.a_log[h]) * dt);
       b = dt;
+    }
+    float qv = 0.f, kv = 0.f;
+    if (tid < D) {
+      qv = src[P.off_q + hg * D + tid] * qscale;
+      kv = src[P.off_k + hg * D + tid];
+      qs[tid] = qv;
+      ks[tid] = kv;
+    }
+    if (tid < Dv) vs[tid] = src[P.off_v + h * Dv + tid];
+    if (MODE == SCAN_MLSTM) {
+      nreg = a * nreg + b * kv;
+      const float pn = wave_sum(nreg * qv);
+      if ((tid & 63) == 0) nred[tid >> 6] = pn;
     }
     __syncthreads();
     float part = 0.f;
@@ -310,18 +440,14 @@ __global__ __launch_bounds__(256) void gated_scan_kernel(ScanParams P, StepRows 
     }
     po[tid] = part;
     __syncthreads();
-    if (tid < Dvp) {
-      float o = 0.f;
-      for (int gg = 0; gg < NG; ++gg) o += po[gg * Dvp + tid];
-      os[tid] = o;
-    }
-    __syncthreads();
     if (tid < Dv) {
+      float o = 0.f;
+      for (int gg = 0; gg < NG; ++gg) o += po[gg * Dv + tid];
       float y;
       if (MODE == SCAN_MLSTM)
-        y = os[tid] / (fmaxf(fabsf(os[Dv]), expf(-m)) + 1e-6f);
+        y = o / (fmaxf(fabsf(nred[0] + nred[1] + nred[2] + nred[3]), expf(-m)) + 1e-6f);
       else
-        y = (os[tid] + P.d_skip[h] * vs[tid]) * silu(row[P.off_g + h * Dv + tid]);
+        y = (o + P.d_skip[h] * vs[tid]) * silu(row[P.off_g + h * Dv + tid]);
       P.y[(long long)r * P.ld_y + h * Dv + tid] = y;
     }
     __syncthreads();
@@ -329,25 +455,22 @@ __global__ __launch_bounds__(256) void gated_scan_kernel(ScanParams P, StepRows 
 #pragma unroll
   for (int ii = 0; ii < MAXI; ++ii) {
     const int i = g + ii * NG;
-    if (act && i < D) {
-      if (j < Dv)
-        S0[(long long)i * Dv + j] = S[ii];
-      else
-        nvec[i] = S[ii];
-    }
+    if (act && i < D) S0[(long long)i * Dv + j] = S[ii];
   }
-  if (MODE == SCAN_MLSTM && tid == 0) *mptr = m;
+  if (MODE == SCAN_MLSTM) {
+    if (tid < D) nvec[tid] = nreg;
+    if (tid == 0) *mptr = m;
+  }
 }
 bool gated_scan_supported(int mode, int D, int Dv) {
-  const int dvp = Dv + (mode == SCAN_MLSTM ? 1 : 0);
-  if (D <= 0 || Dv <= 0 || D > 256 || dvp > 256) return false;
-  const int ng = 256 / dvp;
+  (void)mode;
+  if (D <= 0 || Dv <= 0 || D > 256 || Dv > 256) return false;
+  const int ng = 256 / Dv;
   return (D + ng - 1) / ng <= 64;
 }
 template <int MODE>
 static void launch_gated_scan(const ScanParams& P, const StepRows& R, hipStream_t s) {
-  const int dvp = P.Dv + (MODE == SCAN_MLSTM ? 1 : 0);
-  const int ng = 256 / dvp, ni = (P.D + ng - 1) / ng;
+  const int ng = 256 / P.Dv, ni = (P.D + ng - 1) / ng;
   const dim3 grid(R.B, P.H);
   if (ni <= 8)
     hipLaunchKernelGGL((gated_scan_kernel<MODE, 8>), grid, dim3(256), 0, s, P, R);
@@ -360,7 +483,7 @@ static void launch_gated_scan(const ScanParams& P, const StepRows& R, hipStream_
 }
 void gated_scan(const ScanParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.proj && P.state && P.y && P.H > 0 && P.G > 0 && P.H % P.G == 0 && gated_scan_supported(P.mode, P.D, P.Dv),
-        "gated scan: operands or head sizes (key size <= 256, value size <= 255, state within the registers)");
+        "gated scan: operands or head sizes (key and value size <= 256, state within the registers)");
   if (P.mode == SCAN_MLSTM) {
     check(P.i_b && P.f_b && P.cap > 0.f && P.G == P.H, "gated scan: mLSTM gate operands");
     launch_gated_scan<SCAN_MLSTM>(P, R, s);
@@ -369,6 +492,308 @@ void gated_scan(const ScanParams& P, const StepRows& R, hipStream_t s) {
     launch_gated_scan<SCAN_SSD>(P, R, s);
   }
   launched("gated_scan");
+}
+
+// ---- prompt portions: the same recurrence in chunks of SC tokens, as the chunked retention but with per-row decays.
+// With l_s = ln a_s and L_t = l_0 + ... + l_t inside a chunk of n tokens that starts from state S,
+//   A[t][s] = (q_t . k_s) exp(L_t - L_s) b_s for s <= t,   o_t = exp(L_t) S^T q_t + sum_s A[t][s] v_s,
+//   U = sum_s exp(L_(n-1) - L_s) b_s k_s v_s^T,              S <- exp(L_(n-1)) S + U,
+// all in float32 on the vector ALUs, over the host-built chunk table {first row, rows, state slot, flags}:
+//   0. per (row, head) coefficients {l, b, m}: gated_coef_*                       (the mLSTM's running maximum is a
+//      scan of x -> max(x + f, i), composed over a wave's 64 rows at a time)
+//   1. every chunk's U and its total log decay, chunks in parallel                (gated_u_kernel)
+//   2. the scan over each sequence's chunks, one thread per state element        (gated_chunk_scan_kernel)
+//   3. every chunk's outputs from its incoming state, in parallel                (gated_out_kernel)
+// The mLSTM's normaliser is column Dv of the state here too; its raw outputs [B][H][Dv + 1] are finished by
+// mlstm_finish_kernel (the division, the per-head unit RMS, the norm's weight, the output gate).
+constexpr int SC = 32;
+int gated_chunk_rows() { return SC; }
+bool gated_chunk_supported(int mode, int D, int Dv) { return D > 0 && D <= 128 && Dv > 0 && Dv + (mode == SCAN_MLSTM ? 1 : 0) <= 256; }
+
+__global__ __launch_bounds__(256) void gated_coef_ssd_kernel(ScanParams P, int B, float* __restrict__ coef) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= B * P.H) return;
+  const int r = idx / P.H, h = idx % P.H;
+  const float dt = softplusf(P.proj[(long long)r * P.ld + P.off_i + h] + P.dt_bias[h]);
+  coef[(long long)idx * 3] = -expf(P.a_log[h]) * dt;
+  coef[(long long)idx * 3 + 1] = dt;
+  coef[(long long)idx * 3 + 2] = 0.f;
+}
+// one wave per (sequence segment, head); lanes take 64 consecutive rows, the running maximum crosses them as the
+// composition of the rows' maps x -> max(x + c, d): (c1, d1) then (c2, d2) = (c1 + c2, max(d1 + c2, d2))
+__global__ __launch_bounds__(256) void gated_coef_mlstm_kernel(ScanParams P, StepRows R, float* __restrict__ coef) {
+  const int r0 = blockIdx.x, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int seq = R.q_seq[r0];
+  if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;
+  if (h >= P.H) return;
+  float* mptr = P.state + (long long)seq * P.state_stride + (long long)P.H * P.D * (P.Dv + 1) + h;
+  float m_in = *mptr;
+  for (int t0 = r0; t0 < R.B; t0 += 64) {
+    const int r = t0 + lane;
+    const bool valid = r < R.B && R.q_seq[r] == seq;
+    float c = 0.f, d = -INFINITY, ig = 0.f, fg = 0.f;
+    if (valid) {
+      const float* row = P.proj + (long long)r * P.ld;
+      ig = P.cap * tanhf((row[P.off_i + h] + P.i_b[h]) / P.cap);
+      fg = logsigmoidf(P.cap * tanhf((row[P.off_f + h] + P.f_b[h]) / P.cap));
+      c = fg;
+      d = ig;
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {  // inclusive scan of the composed maps
+      const float pc = __shfl_up(c, off, 64), pd = __shfl_up(d, off, 64);
+      if (lane >= off) {
+        d = fmaxf(pd + c, d);
+        c = pc + c;
+      }
+    }
+    const float m = fmaxf(m_in + c, d);                    // the running maximum after this lane's row
+    float mp = __shfl_up(m, 1, 64);
+    if (lane == 0) mp = m_in;
+    if (valid) {
+      float* o = coef + ((long long)r * P.H + h) * 3;
+      o[0] = fg + mp - m;
+      o[1] = expf(ig - m);
+      o[2] = m;
+    }
+    const unsigned long long mask = __ballot(valid);
+    const int cnt = __popcll(mask);
+    if (cnt == 0) break;
+    m_in = __shfl(m, cnt - 1, 64);
+    if (cnt < 64) break;
+  }
+  if (lane == 0) *mptr = m_in;
+}
+// q (scaled for the mLSTM) and k rows of a chunk into LDS; rows past cn and dims past D zero
+template <int MODE, int MAXD, bool WITH_Q>
+__device__ __forceinline__ void stage_qk_gated(const ScanParams& P, int row0, int cn, int hg, float (*Qs)[MAXD],
+                                               float (*Ks)[MAXD + 4]) {
+  const float qscale = MODE == SCAN_MLSTM ? 1.f / sqrtf((float)P.D) : 1.f;
+  for (int idx = threadIdx.x; idx < SC * MAXD; idx += 256) {
+    const int c = idx / MAXD, d = idx % MAXD;
+    float qv = 0.f, kv = 0.f;
+    if (c < cn && d < P.D) {
+      const float* src = MODE == SCAN_MLSTM ? P.proj + (long long)(row0 + c) * P.ld : P.conv + (long long)(row0 + c) * P.ld_conv;
+      kv = src[P.off_k + hg * P.D + d];
+      if (WITH_Q) qv = src[P.off_q + hg * P.D + d] * qscale;
+    }
+    if (WITH_Q) Qs[c][d] = qv;
+    Ks[c][d] = kv;
+  }
+}
+// value columns jb * 64 .. + 63 of a chunk's rows; the mLSTM's column Dv is 1 (the normaliser)
+template <int MODE>
+__device__ __forceinline__ void stage_v_gated(const ScanParams& P, int row0, int cn, int h, int jb, float (*Vs)[64]) {
+  for (int idx = threadIdx.x; idx < SC * 64; idx += 256) {
+    const int c = idx >> 6, col = jb * 64 + (idx & 63);
+    float v = 0.f;
+    if (c < cn) {
+      const float* src = MODE == SCAN_MLSTM ? P.proj + (long long)(row0 + c) * P.ld : P.conv + (long long)(row0 + c) * P.ld_conv;
+      if (col < P.Dv)
+        v = src[P.off_v + h * P.Dv + col];
+      else if (MODE == SCAN_MLSTM && col == P.Dv)
+        v = 1.f;
+    }
+    Vs[c][idx & 63] = v;
+  }
+}
+// Lc[t] = l_0 + ... + l_t and bw[t] = b_t of the chunk's rows (Lc past cn stays at its last value)
+__device__ __forceinline__ void stage_coef(const ScanParams& P, const float* coef, int row0, int cn, int h, float* Lc, float* bw) {
+  if (threadIdx.x < SC) {
+    const int t = threadIdx.x;
+    const float* c = coef + ((long long)(row0 + min(t, cn - 1)) * P.H + h) * 3;
+    Lc[t] = t < cn ? c[0] : 0.f;
+    bw[t] = t < cn ? c[1] : 0.f;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float acc = 0.f;
+    for (int t = 0; t < SC; ++t) {
+      acc += Lc[t];
+      Lc[t] = acc;
+    }
+  }
+  __syncthreads();
+}
+template <int MODE, int MAXD>
+__global__ __launch_bounds__(256) void gated_u_kernel(ScanParams P, const int* __restrict__ chunks, const float* __restrict__ coef,
+                                                      float* __restrict__ U, long long u_stride, float* __restrict__ ctot,
+                                                      int NJ) {
+  __shared__ __attribute__((aligned(16))) float Ks[SC][MAXD + 4];
+  __shared__ float Vs[SC][64];
+  __shared__ float Lc[SC], bw[SC];
+  const int c = blockIdx.x, h = blockIdx.y / NJ, jb = blockIdx.y % NJ, tid = threadIdx.x;
+  const int row0 = chunks[4 * c], cn = chunks[4 * c + 1];
+  const int Dvp = P.Dv + (MODE == SCAN_MLSTM ? 1 : 0);
+  const int j = tid & 63, g4 = tid >> 6, col = jb * 64 + j;
+  stage_coef(P, coef, row0, cn, h, Lc, bw);
+  stage_qk_gated<MODE, MAXD, false>(P, row0, cn, h / (P.H / P.G), nullptr, Ks);
+  stage_v_gated<MODE>(P, row0, cn, h, jb, Vs);
+  __syncthreads();
+  if (jb == 0 && tid == 0) ctot[(long long)c * P.H + h] = Lc[cn - 1];
+  float u[MAXD / 4];
+#pragma unroll
+  for (int ii = 0; ii < MAXD / 4; ++ii) u[ii] = 0.f;
+  for (int sx = 0; sx < cn; ++sx) {
+    const float vv = Vs[sx][j] * (expf(Lc[cn - 1] - Lc[sx]) * bw[sx]);
+#pragma unroll
+    for (int ii = 0; ii < MAXD / 4; ++ii) u[ii] += Ks[sx][g4 + 4 * ii] * vv;
+  }
+  if (col < Dvp) {
+    float* out = U + c * u_stride + (long long)h * P.D * Dvp;
+#pragma unroll
+    for (int ii = 0; ii < MAXD / 4; ++ii) {
+      const int i = g4 + 4 * ii;
+      if (i < P.D) out[(long long)i * Dvp + col] = u[ii];
+    }
+  }
+}
+template <int MODE>
+__global__ __launch_bounds__(256) void gated_chunk_scan_kernel(ScanParams P, const int* __restrict__ chunks, int nchunks,
+                                                               const float* __restrict__ U, float* __restrict__ Sin,
+                                                               long long u_stride, const float* __restrict__ ctot) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int Dvp = P.Dv + (MODE == SCAN_MLSTM ? 1 : 0);
+  const long long per_head = (long long)P.D * Dvp;
+  if (e >= P.H * per_head) return;
+  const int h = (int)(e / per_head), i = (int)(e % per_head) / Dvp, j = (int)(e % per_head) % Dvp;
+  // where this element lives in a slot's state: S [H][D][Dv], then (mLSTM) the normaliser [H][D]
+  const long long at = j < P.Dv ? ((long long)h * P.D + i) * P.Dv + j : (long long)P.H * P.D * P.Dv + (long long)h * P.D + i;
+  float S = 0.f;
+  for (int c = 0; c < nchunks; ++c) {
+    const int slot = chunks[4 * c + 2], flags = chunks[4 * c + 3];
+    float* st_e = P.state + (long long)slot * P.state_stride + at;
+    if (flags & 1) S = *st_e;
+    Sin[c * u_stride + e] = S;
+    S = expf(ctot[(long long)c * P.H + h]) * S + U[c * u_stride + e];
+    if (flags & 2) *st_e = S;
+  }
+}
+template <int MODE, int MAXD>
+__global__ __launch_bounds__(256) void gated_out_kernel(ScanParams P, const int* __restrict__ chunks, const float* __restrict__ coef,
+                                                        const float* __restrict__ Sin, long long u_stride,
+                                                        float* __restrict__ raw, int ld_raw, int NJ) {
+  __shared__ __attribute__((aligned(16))) float Qs[SC][MAXD];
+  __shared__ __attribute__((aligned(16))) float Ks[SC][MAXD + 4];
+  __shared__ float Vs[SC][64];
+  __shared__ float As[SC][SC + 1];
+  __shared__ float Lc[SC], bw[SC];
+  const int c = blockIdx.x, h = blockIdx.y / NJ, jb = blockIdx.y % NJ, tid = threadIdx.x;
+  const int row0 = chunks[4 * c], cn = chunks[4 * c + 1];
+  const int D = P.D, Dv = P.Dv;
+  const int Dvp = Dv + (MODE == SCAN_MLSTM ? 1 : 0);
+  const int j = tid & 63, g4 = tid >> 6, col = jb * 64 + j;
+  const bool colok = col < Dvp;
+  float S[MAXD];
+  const float* sin_base = Sin + c * u_stride + (long long)h * D * Dvp;
+#pragma unroll
+  for (int i = 0; i < MAXD; ++i) S[i] = (colok && i < D) ? sin_base[(long long)i * Dvp + col] : 0.f;
+  stage_coef(P, coef, row0, cn, h, Lc, bw);
+  stage_qk_gated<MODE, MAXD, true>(P, row0, cn, h / (P.H / P.G), Qs, Ks);
+  stage_v_gated<MODE>(P, row0, cn, h, jb, Vs);
+  __syncthreads();
+#pragma unroll
+  for (int kx = 0; kx < SC * SC / 256; ++kx) {
+    const int t = (tid >> 5) + 8 * kx, sx = tid & 31;
+    float dot = 0.f;
+    if (sx <= t && t < cn) {
+#pragma unroll
+      for (int i4 = 0; i4 < MAXD / 4; ++i4) {
+        const f32x4 qa = *(const f32x4*)&Qs[t][4 * i4], kb = *(const f32x4*)&Ks[sx][4 * i4];
+        dot += qa[0] * kb[0] + qa[1] * kb[1] + qa[2] * kb[2] + qa[3] * kb[3];
+      }
+      dot *= expf(Lc[t] - Lc[sx]) * bw[sx];
+    }
+    As[t][sx] = dot;
+  }
+  __syncthreads();
+  for (int t = g4; t < cn; t += 4) {
+    float inter = 0.f;
+#pragma unroll
+    for (int i4 = 0; i4 < MAXD / 4; ++i4) {
+      const f32x4 qa = *(const f32x4*)&Qs[t][4 * i4];
+      inter += qa[0] * S[4 * i4] + qa[1] * S[4 * i4 + 1] + qa[2] * S[4 * i4 + 2] + qa[3] * S[4 * i4 + 3];
+    }
+    float intra = 0.f;
+#pragma unroll
+    for (int sx = 0; sx < SC; ++sx) intra += As[t][sx] * Vs[sx][j];  // As is zero above the diagonal
+    if (colok) {
+      const float o = expf(Lc[t]) * inter + intra;
+      const long long r = row0 + t;
+      if (MODE == SCAN_MLSTM)
+        raw[r * ld_raw + h * Dvp + col] = o;
+      else
+        P.y[r * P.ld_y + h * Dv + col] = (o + P.d_skip[h] * Vs[t][j]) * silu(P.proj[r * P.ld + P.off_g + h * Dv + col]);
+    }
+  }
+}
+// mLSTM: y = o / (max(|n . q|, exp(-m)) + 1e-6), divided by its root mean square over the head, times the norm's
+// weight and the sigmoid output gate; one wave per (row, head)
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_finish_kernel(ScanParams P, int B, const float* __restrict__ raw, int ld_raw,
+                                                           const float* __restrict__ coef, const float* __restrict__ w, float eps,
+                                                           T* __restrict__ out, int ld_out) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= B * P.H) return;
+  const int b = item / P.H, h = item % P.H, Dv = P.Dv;
+  const float* o = raw + (long long)b * ld_raw + h * (Dv + 1);
+  const float den = fmaxf(fabsf(o[Dv]), expf(-coef[(long long)item * 3 + 2])) + 1e-6f;
+  float sq = 0.f;
+  for (int jx = lane; jx < Dv; jx += 64) sq += (o[jx] / den) * (o[jx] / den);
+  const float rs = 1.f / sqrtf(wave_sum(sq) / (float)Dv + eps);
+  const float* gate = P.proj + (long long)b * P.ld + P.off_g + h * Dv;
+  for (int jx = lane; jx < Dv; jx += 64)
+    st(out + (long long)b * ld_out + h * Dv + jx, o[jx] / den * rs * w[h * Dv + jx] * sigmoidf(gate[jx]));
+}
+template <int MODE, int MAXD>
+static void launch_gated_chunked(const ScanParams& P, const StepRows& R, const ScanChunkWs& W, hipStream_t s) {
+  const int Dvp = P.Dv + (MODE == SCAN_MLSTM ? 1 : 0), NJ = (Dvp + 63) / 64;
+  const dim3 grid(W.nchunks, P.H * NJ);
+  hipLaunchKernelGGL((gated_u_kernel<MODE, MAXD>), grid, dim3(256), 0, s, P, W.chunks, W.coef, W.U, W.u_stride, W.ctot, NJ);
+  launched("gated_u");
+  const long long elems = (long long)P.H * P.D * Dvp;
+  hipLaunchKernelGGL(gated_chunk_scan_kernel<MODE>, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, s, P, W.chunks, W.nchunks,
+                     W.U, W.Sin, W.u_stride, W.ctot);
+  launched("gated_chunk_scan");
+  hipLaunchKernelGGL((gated_out_kernel<MODE, MAXD>), grid, dim3(256), 0, s, P, W.chunks, W.coef, W.Sin, W.u_stride, W.raw,
+                     W.ld_raw, NJ);
+  launched("gated_out");
+}
+void gated_scan_chunked(const ScanParams& P, const StepRows& R, const ScanChunkWs& W, const float* norm_w, float eps, void* out,
+                        int ld_out, int f32, hipStream_t s) {
+  const int Dvp = P.Dv + (P.mode == SCAN_MLSTM ? 1 : 0);
+  check(R.B > 0 && P.proj && P.state && P.H > 0 && P.G > 0 && P.H % P.G == 0 && gated_chunk_supported(P.mode, P.D, P.Dv),
+        "chunked gated scan: key size <= 128, value size <= 255");
+  check(W.chunks && W.nchunks > 0 && W.nchunks <= W.max_chunks && W.U && W.Sin && W.coef && W.ctot &&
+            W.u_stride >= (long long)P.H * P.D * Dvp,
+        "chunked gated scan: chunk table or workspace");
+  if (P.mode == SCAN_MLSTM) {
+    check(P.i_b && P.f_b && P.cap > 0.f && P.G == P.H && W.raw && W.ld_raw >= P.H * Dvp && norm_w && out, "chunked mLSTM operands");
+    hipLaunchKernelGGL(gated_coef_mlstm_kernel, dim3(R.B, (P.H + 3) / 4), dim3(256), 0, s, P, R, W.coef);
+    launched("gated_coef_mlstm");
+    if (P.D <= 64)
+      launch_gated_chunked<SCAN_MLSTM, 64>(P, R, W, s);
+    else
+      launch_gated_chunked<SCAN_MLSTM, 128>(P, R, W, s);
+    const dim3 g2((R.B * P.H + 3) / 4);
+    if (f32)
+      hipLaunchKernelGGL(mlstm_finish_kernel<float>, g2, dim3(256), 0, s, P, R.B, W.raw, W.ld_raw, W.coef, norm_w, eps, (float*)out,
+                         ld_out);
+    else
+      hipLaunchKernelGGL(mlstm_finish_kernel<bf16>, g2, dim3(256), 0, s, P, R.B, W.raw, W.ld_raw, W.coef, norm_w, eps, (bf16*)out,
+                         ld_out);
+    launched("mlstm_finish");
+  } else {
+    check(P.conv && P.dt_bias && P.a_log && P.d_skip && P.y, "chunked state space operands");
+    hipLaunchKernelGGL(gated_coef_ssd_kernel, dim3((R.B * P.H + 255) / 256), dim3(256), 0, s, P, R.B, W.coef);
+    launched("gated_coef_ssd");
+    if (P.D <= 64)
+      launch_gated_chunked<SCAN_SSD, 64>(P, R, W, s);
+    else
+      launch_gated_chunked<SCAN_SSD, 128>(P, R, W, s);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ grouped RMS norm

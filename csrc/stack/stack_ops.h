@@ -194,6 +194,8 @@ struct LatentParams {
   float eps;
   const void* w_uk;     // [H * D][C]
   const void* w_uvT;    // [H][C][Dv]
+  const void* w_ukT;    // [H][C][D]   (or null) the layouts the few-row kernels read
+  const void* w_uv;     // [H * Dv][C] (or null)
   void* cache;          // [blocks][1][bs][C + R] matrix dtype
   float* qa;            // [B][ld_qa]: per head [W_uk_h^T q_plain | rotated q part] (the attention's queries)
   int ld_qa;
@@ -244,6 +246,27 @@ struct ScanParams {
 };
 void gated_scan(const ScanParams& P, const StepRows& R, hipStream_t s);
 bool gated_scan_supported(int mode, int D, int Dv);
+// the same recurrence in chunks (prompt portions) over the host-built chunk table of the chunked retention
+// ({first row, rows <= gated_chunk_rows(), state slot, flags}); U and Sin hold one state per chunk
+// ([H][D][Dv (+ 1 for the mLSTM's normaliser)]), coef [B][H][3] the rows' {ln a, b, m}, ctot [chunks][H] the chunks'
+// summed ln a, raw [B][ld_raw] the mLSTM's outputs before their division ([H][Dv + 1]). SCAN_SSD leaves P.y as
+// gated_scan does; SCAN_MLSTM goes on to the finished mixer output `out` (division, per-head unit RMS, norm_w, the
+// sigmoid gate at P.off_g), matrix dtype.
+struct ScanChunkWs {
+  const int* chunks;
+  int nchunks, max_chunks;
+  float* U;
+  float* Sin;
+  long long u_stride;
+  float* coef;
+  float* ctot;
+  float* raw;
+  int ld_raw;
+};
+void gated_scan_chunked(const ScanParams& P, const StepRows& R, const ScanChunkWs& W, const float* norm_w, float eps, void* out,
+                        int ld_out, int f32, hipStream_t s);
+int gated_chunk_rows();
+bool gated_chunk_supported(int mode, int D, int Dv);
 // out = y / rms(y over each of `groups` equal parts) * w * (gate ? sigmoid(gate) : 1), matrix dtype
 void group_rms_cast(const float* y, int ld_y, int rows, int n, int groups, const float* w, float eps, const float* gate,
                     int ld_gate, void* out, int ld_out, int f32, hipStream_t s);

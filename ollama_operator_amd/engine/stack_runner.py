@@ -66,7 +66,7 @@ class StackExec:
                     self._f64.append(L["inv_freq"].double().contiguous())
                 d.update(norm2_w=p(L.get("norm2_w")), norm2_b=p(L.get("norm2_b")), w_ff=p(L.get("w_ff")), n_ff=L["n_ff"],
                          rot_dim=m.rot_dim, kv_rank=m.kv_rank, dkv_norm=p(L.get("dkv_norm")), w_uk=p(L.get("w_uk")),
-                         w_uvT=p(L.get("w_uvT")), sink=p(L.get("sink")), gate_cap=m.gate_cap, i_b=p(L.get("i_b")),
+                         w_uvT=p(L.get("w_uvT")), w_ukT=p(L.get("w_ukT")), w_uv=p(L.get("w_uv")), sink=p(L.get("sink")), gate_cap=m.gate_cap, i_b=p(L.get("i_b")),
                          f_b=p(L.get("f_b")), mnorm=p(L.get("mnorm")), state=m.state, groups=m.groups, conv=m.conv,
                          norm_groups=m.norm_groups, conv_w=p(L.get("conv_w")), conv_b=p(L.get("conv_b")),
                          dt_bias=p(L.get("dt_bias")), a_log=p(L.get("a_log")), d_skip=p(L.get("d_skip")),
@@ -82,7 +82,8 @@ class StackExec:
                              split_ws=p(r.split_ws), split_ws_floats=r.split_ws.numel(),
                              ret_chunks=p(r.d_chunks), ret_max_chunks=r.d_chunks.shape[0], ret_u=p(r.ret_u),
                              ret_sin=p(r.ret_sin), ret_u_stride=r.ret_u.shape[1], cbuf=p(r.cbuf), ld_cbuf=r.cbuf.shape[1],
-                             lat=p(r.latbuf), ld_lat=r.latbuf.shape[1], idw=p(r.idw),
+                             lat=p(r.latbuf), ld_lat=r.latbuf.shape[1], idw=p(r.idw), coef=p(r.scan_coef),
+                             ld_coef=(r.scan_coef.shape[1] if r.scan_coef is not None else 0), ctot=p(r.scan_ctot),
                              **{"moe_" + k: (v if isinstance(v, int) else p(v)) for k, v in r.moe_ws.items()}))
         e.set_inputs(dict(tokens=p(r.d_tokens), pos=p(r.d_pos), slot=p(r.d_slot), q_len=p(r.d_qlen),
                           q_seq=p(r.d_qseq), block_table=p(r.d_block_table), max_blocks=r.max_blocks,
@@ -203,13 +204,19 @@ class StackRunner(Runner):
         self.ew = torch.zeros(max_batch, top, **f32)
         self.sgate = torch.zeros(max_batch, **f32)
         self.lbuf = torch.zeros(max_batch, E, **tt)
-        self.obuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **f32)  # retention, before its norm
+        # state mixers' outputs before their norm (the mLSTM's with its normaliser's column per head)
+        self.obuf = torch.zeros(max_batch, max(s.mixer.heads * (s.mixer.vdim + (s.mixer.kind == MIX_MLSTM)) for s in cfg.layers), **f32)
         # chunked retention of prompt portions: the chunk table and one state per chunk (its U, its incoming state)
-        rets = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_RETENTION]
+        rets = [s.mixer for s in cfg.layers if s.mixer.kind in (MIX_RETENTION, MIX_MLSTM, MIX_MAMBA2)]
         n_ch = max_batch // 32 + max_seqs + 1 if rets and max_batch > 16 else 1
         self.d_chunks = torch.zeros(n_ch, 4, **i32)
         self.d_tiles = torch.zeros(max_batch // 32 + max_seqs + 1, 2, **i32)  # attention query tiles of a step
-        self.ret_u = torch.zeros(n_ch, max([m.heads * m.dim * m.vdim for m in rets], default=1) if n_ch > 1 else 1, **f32)
+        self.ret_u = torch.zeros(n_ch, max([m.heads * m.dim * (m.vdim + (m.kind == MIX_MLSTM)) for m in rets], default=1)
+                                 if n_ch > 1 else 1, **f32)
+        # chunked gated scans: the rows' {ln decay, input weight, running maximum} per head, the chunks' summed ln decay
+        hmax = max([m.heads for m in rets if m.kind != MIX_RETENTION], default=0) if n_ch > 1 else 0
+        self.scan_coef = torch.zeros(max_batch, 3 * hmax, **f32) if hmax else None
+        self.scan_ctot = torch.zeros(n_ch, hmax, **f32) if hmax else None
         self.ret_sin = torch.zeros_like(self.ret_u)
         # decode attention over long contexts: partials {maximum, sum, output} of up to 16 splits per (row, head)
         hv = max([s.mixer.heads * (s.mixer.vdim + 2) for s in cfg.layers if s.mixer.kind == MIX_ATTENTION] +

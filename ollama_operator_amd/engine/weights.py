@@ -485,7 +485,8 @@ class StackWeights:
         matrices that read the stream are one stacked `w_in`; the feed-forward reads the UPDATED stream, so its
         input matrices (router | shared gate | shared up, or the dense up) are a second stack `w_ff`.
         Latent attention keeps W_uk as stored ([H * dim][rank]: the query is folded onto the latent through it)
-        and W_uv transposed per head ([H][rank][vdim]: the latent-space output is expanded through it)."""
+        and W_uv transposed per head ([H][rank][vdim]: the latent-space output is expanded through it), and
+        the other layout of both for steps of a few rows."""
         from ..models.config import FF_DENSE, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM
         get, mat, vec = self._get, self._mat, self._vec
         E, m, f, dev = self.cfg.n_embd, spec.mixer, spec.mlp, self.device
@@ -497,6 +498,9 @@ class StackWeights:
             L["dkv_norm"] = vec(get(p + "mix.dkv.norm", (C,)))
             L["w_uk"] = mat(get(p + "mix.uk", (H * D, C)))
             L["w_uvT"] = mat(get(p + "mix.uv", (H * Dv, C)).view(H, Dv, C).transpose(1, 2).reshape(H * C, Dv))
+            # the other layout of each, for steps of a few rows (one weight row per wave, read along its length)
+            L["w_ukT"] = mat(get(p + "mix.uk", (H * D, C)).view(H, D, C).transpose(1, 2).reshape(H * C, D))
+            L["w_uv"] = mat(get(p + "mix.uv", (H * Dv, C)))
             L["sink"] = vec(get(p + "mix.sink", (H,)))
             L["inv_freq"] = (torch.from_numpy(rope_inv_freq(m.rot_dims, m.rot_base)).to(dev) if m.rot_dims else None)
         elif m.kind == MIX_MLSTM:

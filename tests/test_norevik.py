@@ -58,6 +58,7 @@ MECHANISMS = {
     "latent_all_rotated": [(nc.latent(), None)],
     "latent_part_rotated_one_head": [(nc.latent(heads=1, dim=24, rot_dim=10, vdim=7, kv_rank=13, rot_dims=6), None)],
     "latent_no_rotation": [(nc.latent(rot_dim=4, rot_dims=0), None)],
+    "latent_no_shared_key_part": [(nc.latent(heads=2, dim=16, rot_dim=0, vdim=8, kv_rank=16), None)],
     "mlstm": [(nc.mlstm(), None)],
     "mlstm_tight_cap_one_head": [(nc.mlstm(heads=1, dim=20, vdim=3, cap=1.5), None)],
     "mamba2": [(nc.mamba(), None)],
