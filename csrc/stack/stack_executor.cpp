@@ -111,7 +111,10 @@ void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
     // row and whose value is the row's first C elements
     AttnParams A{ws.cbuf, ws.ld_cbuf, 0, 0, 0, L.heads, 1, W, C, L.scale, 0.f, 0.f, 1, r.kc, r.kc, ws.lat, ws.ld_lat, f32,
                  n_splits, ws.split_ws, ws.split_ws_floats, W, W, L.sink};
-    attention(A, R, s);
+    if (B > SMALL_B && n_tiles > 0 && tiles && flash_prefill_supported(A))
+      flash_prefill(A, R, tiles, n_tiles, s);  // prompt portions: query tiles on the matrix cores
+    else
+      attention(A, R, s);
     latent_expand(P, B, s);
   } else if (L.kind == 3) {
     ScanParams P{};

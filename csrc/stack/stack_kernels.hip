@@ -1015,6 +1015,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   const float inv_cap = P.softcap != 0.f ? 1.f / P.softcap : 0.f;
   const uint16_t* kc = (const uint16_t*)P.kc;
   const uint16_t* vc = (const uint16_t*)P.vc;
+  const long long ldk = P.ldk ? P.ldk : D, ldv = P.ldv ? P.ldv : DV;  // row strides of the pools
   // The K fragments and V rows of the NEXT key group are requested before the current group is multiplied, so a
   // group's global round trip passes behind the previous group's products and softmax.
   constexpr int CH = DV / 8;            // 16-byte pieces per V row
@@ -1024,7 +1025,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
     {
       const int key = min(t0 + kperm, kmax - 1);
       const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
-      const uint16_t* kr = kc + rowidx * D + 8 * hf;
+      const uint16_t* kr = kc + rowidx * ldk + 8 * hf;
 #pragma unroll
       for (int kk = 0; kk < KD; ++kk) kf_n[kk] = *(const u32x4*)(kr + 16 * kk);
     }
@@ -1033,7 +1034,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
       const int c = lane + 64 * i;
       const int key = min(t0 + c / CH, kmax - 1), seg = c % CH;
       const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
-      vs_n[i] = *(const u32x4*)(vc + rowidx * DV + 8 * seg);
+      vs_n[i] = *(const u32x4*)(vc + rowidx * ldv + 8 * seg);
     }
   };
   fetch(0);
@@ -1120,6 +1121,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   }
   if (q < nrows) {  // register r of tile j: value dim 32 j + (r & 3) + 8 (r >> 2) + 4 hf of this lane's query
     bf16* out = (bf16*)P.out + (long long)qrow * P.ld_out + h * DV;
+    if (P.sink) li += expf(P.sink[h] - mi);  // the sink: a term of the denominator without key or value
     const float inv = 1.f / li;
 #pragma unroll
     for (int j = 0; j < NV; ++j)
@@ -1127,22 +1129,28 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
       for (int r = 0; r < 16; ++r) st(out + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hf, o[j][r] * inv);
   }
 }
+// (key size / 16, value size / 32) the kernel is built for: equal key and value sizes 64 / 96 / 128, and the rows of
+// latent attention (key = latent + shared rotated part, value = the latent)
+#define FLASH_SHAPES(X) X(4, 2) X(6, 3) X(8, 4) X(7, 3) X(8, 3) X(9, 4) X(10, 4) X(12, 5) X(14, 6) X(16, 6) X(16, 7)
 bool flash_prefill_supported(const AttnParams& P) {
-  return !P.f32 && !P.sink && !P.ldk && !P.ldv && P.D == P.Dv && (P.D == 64 || P.D == 96 || P.D == 128) && P.ld % 4 == 0 && P.off_q % 4 == 0 &&
+  bool shape = false;
+#define FLASH_HAS(KD, NV) shape |= P.D == 16 * KD && P.Dv == 32 * NV;
+  FLASH_SHAPES(FLASH_HAS)
+#undef FLASH_HAS
+  const int ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
+  return !P.f32 && shape && ldk % 8 == 0 && ldv % 8 == 0 && P.ld % 4 == 0 && P.off_q % 4 == 0 && (P.H * P.D) % 4 == 0 &&
          ((uintptr_t)P.proj & 15) == 0 && ((uintptr_t)P.kc & 15) == 0 && ((uintptr_t)P.vc & 15) == 0;
 }
 void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s) {
   check(flash_prefill_supported(P) && tiles && ntiles > 0 && P.G > 0 && P.H % P.G == 0 && P.out, "flash prefill: operands");
   dim3 grid(ntiles, P.H);
-  if (P.D == 64)
-    hipLaunchKernelGGL((flash_prefill_kernel<4, 2>), grid, dim3(64), 0, s, P, R, tiles);
-  else if (P.D == 96)
-    hipLaunchKernelGGL((flash_prefill_kernel<6, 3>), grid, dim3(64), 0, s, P, R, tiles);
-  else
-    hipLaunchKernelGGL((flash_prefill_kernel<8, 4>), grid, dim3(64), 0, s, P, R, tiles);
+#define FLASH_LAUNCH(KD, NV)                  \
+  if (P.D == 16 * KD && P.Dv == 32 * NV)      \
+    hipLaunchKernelGGL((flash_prefill_kernel<KD, NV>), grid, dim3(64), 0, s, P, R, tiles);
+  FLASH_SHAPES(FLASH_LAUNCH)
+#undef FLASH_LAUNCH
   launched("flash_prefill");
 }
-
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && P.out,
         "attention: head sizes up to 256, heads a multiple of key/value heads");

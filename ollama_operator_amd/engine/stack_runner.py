@@ -66,7 +66,8 @@ class StackExec:
                     self._f64.append(L["inv_freq"].double().contiguous())
                 d.update(norm2_w=p(L.get("norm2_w")), norm2_b=p(L.get("norm2_b")), w_ff=p(L.get("w_ff")), n_ff=L["n_ff"],
                          rot_dim=m.rot_dim, kv_rank=m.kv_rank, dkv_norm=p(L.get("dkv_norm")), w_uk=p(L.get("w_uk")),
-                         w_uvT=p(L.get("w_uvT")), w_ukT=p(L.get("w_ukT")), w_uv=p(L.get("w_uv")), sink=p(L.get("sink")), gate_cap=m.gate_cap, i_b=p(L.get("i_b")),
+                         w_uvT=p(L.get("w_uvT")), w_ukT=p(L.get("w_ukT")), w_uv=p(L.get("w_uv")), sink=p(L.get("sink")),
+                         gate_cap=m.gate_cap, i_b=p(L.get("i_b")),
                          f_b=p(L.get("f_b")), mnorm=p(L.get("mnorm")), state=m.state, groups=m.groups, conv=m.conv,
                          norm_groups=m.norm_groups, conv_w=p(L.get("conv_w")), conv_b=p(L.get("conv_b")),
                          dt_bias=p(L.get("dt_bias")), a_log=p(L.get("a_log")), d_skip=p(L.get("d_skip")),

@@ -288,10 +288,12 @@ def test_memories_that_last_and_gates_at_their_limits(tmp_path, device):
 def test_other_sizes(tmp_path, device, dtype):
     """A width, head sizes and expert sizes that are not multiples of 8 (no vector loads), more rows than one
     tile, a vocabulary wider than a tile, eps and embedding scale of their own, every group kept, top 4."""
-    layers = [(nc.latent(heads=5, dim=12, rot_dim=6, vdim=10, kv_rank=18, scale=0.4, rot_dims=4), nc.moe(experts=9, top=4, ff=20, shared_ff=12, identity=1, groups=(5, 3))),
+    layers = [(nc.latent(heads=5, dim=12, rot_dim=6, vdim=10, kv_rank=18, scale=0.4, rot_dims=4),
+               nc.moe(experts=9, top=4, ff=20, shared_ff=12, identity=1, groups=(5, 3))),
               (nc.mamba(heads=6, vdim=6, state=10, groups=3, conv=5, norm_groups=2), nc.dense(36)),
               (nc.mlstm(heads=5, dim=6, vdim=14, cap=9.0), nc.moe(experts=3, top=3, ff=12, shared_ff=0, identity=0, groups=(1, 1))),
-              (nc.latent(heads=2, dim=64, rot_dim=32, vdim=64, kv_rank=96, scale=0.1), nc.moe(experts=16, top=2, ff=64, shared_ff=64, identity=0, groups=(4, 2)))]
+              (nc.latent(heads=2, dim=64, rot_dim=32, vdim=64, kv_rank=96, scale=0.1),
+               nc.moe(experts=16, top=2, ff=64, shared_ff=64, identity=0, groups=(4, 2)))]
     m = nc.Model(tmp_path, nc.config(layers, width=52, vocab=300, eps=1e-3, embed_scale=0.7), seed=17)
     toks = nc.tokens(90, 300, seed=18)
     want, _ = m.oracle(toks)
@@ -303,7 +305,8 @@ def test_other_sizes(tmp_path, device, dtype):
 def test_matrix_core_sizes(tmp_path, device):
     """Sizes the matrix-core products and vector loads take (multiples of 64), in bfloat16, with enough rows for the
     grouped routed feed-forward; prompt portion, then single tokens."""
-    layers = [(nc.latent(heads=4, dim=64, rot_dim=32, vdim=64, kv_rank=96, scale=0.1), nc.moe(experts=6, top=2, ff=64, shared_ff=128, identity=2, groups=(2, 1))),
+    layers = [(nc.latent(heads=4, dim=64, rot_dim=32, vdim=64, kv_rank=96, scale=0.1),
+               nc.moe(experts=6, top=2, ff=64, shared_ff=128, identity=2, groups=(2, 1))),
               (nc.mamba(heads=4, vdim=32, state=32, groups=1, conv=4, norm_groups=2), nc.dense(256)),
               (nc.mlstm(heads=2, dim=32, vdim=64, cap=10.0), nc.moe(experts=4, top=2, ff=128, shared_ff=64, identity=0, groups=(1, 1)))]
     m = nc.Model(tmp_path, nc.config(layers, width=128, vocab=256), seed=19)
@@ -391,3 +394,21 @@ def test_gpu_matches_twin_layer_by_layer(std):
         b = nc.layer_trail(std.runner("cuda", dtype), toks)
         for i in range(a.shape[0]):
             assert np.abs(a[i] - b[i]).max() < tol * max(1.0, np.abs(a[i]).max()), f"{dtype}: layer run {i}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rank,rot", [(96, 32), (128, 16)])
+def test_matrix_core_attention_matches_twin(tmp_path, rank, rot):
+    """Latent attention of prompt portions on the matrix cores (bfloat16): one layer, so rounding is not amplified and
+    the comparison is sharp; sinks from dominant to negligible; a portion that starts in the middle of the cache."""
+    m = nc.Model(tmp_path, nc.config([(nc.latent(heads=4, dim=48, rot_dim=rot, vdim=40, kv_rank=rank, scale=0.6), None)],
+                                     width=128, vocab=128), seed=23)
+    m.set_tensor("l0.mix.sink", torch.tensor([12.0, -30.0, 2.0, 5.0]))
+    toks = nc.tokens(230, 128, seed=24)
+    want, _ = m.oracle(toks)
+    a = nc.run_cuts(m.runner("cpu", "bfloat16", max_batch=256), toks, [70, 230])
+    b = nc.run_cuts(m.runner("cuda", "bfloat16", max_batch=256), toks, [70, 230])
+    e = nc.rel_err(b, a)
+    assert np.median(e) < 5e-3 and e.max() < 3e-2, f"HIP against twin: median {np.median(e):.3g}, worst {e.max():.3g}"
+    e = nc.rel_err(b, want)
+    assert np.median(e) < 2e-2 and e.max() < 0.1, f"HIP against the plain implementation: median {np.median(e):.3g}, worst {e.max():.3g}"
