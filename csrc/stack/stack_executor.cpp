@@ -200,12 +200,17 @@ void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
     MoeParams M{ws.proj, ws.ld_proj, L.off_router, 0, L.off_sgate, L.off_sup, B, E, L.experts, L.top, L.ff, L.shared_ff,
                 L.router_b, ws.h, L.w_gu, L.w_down, L.sh_down, ws.eids, ws.ew, ws.ld_top, ws.sgate, ws.hmid, ws.ld_hmid, ws.y,
                 f32, L.identity, L.group_count, L.group_keep, ws.idw};
-    moe_route_scores(M, s);
-    if (B > SMALL_B && ws.moe.gu && moe_grouped_supported(M)) {
-      moe_grouped(M, ws.moe, s);
-    } else {
-      moe_experts(M, s);
+    if (B <= SMALL_B && moe_route_scores_fused_supported(M)) {  // decode steps: routing + activations in one launch
+      moe_route_scores_experts(M, s);
       moe_down(M, s);
+    } else {
+      moe_route_scores(M, s);
+      if (B > SMALL_B && ws.moe.gu && moe_grouped_supported(M)) {
+        moe_grouped(M, ws.moe, s);
+      } else {
+        moe_experts(M, s);
+        moe_down(M, s);
+      }
     }
     if (L.identity) idw = ws.idw;
   }

@@ -1868,7 +1868,7 @@ void moe_fused_small(const MoeParams& P, const void* a, int lda, const void* w_o
 }
 
 static void check_moe(const MoeParams& P) {
-  check(P.B > 0 && P.X > 0 && P.top > 0 && P.top <= P.X && P.top <= MOE_MAX_TOP && P.F > 0 && P.proj && P.h && P.w_gu &&
+  check(P.B > 0 && P.X > 0 && P.top > 0 && P.top <= P.X + P.identity && P.top <= MOE_MAX_TOP && P.F > 0 && P.proj && P.h && P.w_gu &&
             P.w_down && P.eids && P.ew && P.hmid && P.y && P.router_b && P.ld_top >= P.top &&
             P.ld_hmid >= P.top * P.F + P.Fs && (P.Fs == 0 || (P.sh_down && P.sgate)),
         "routed feed-forward: bad operands (top <= 16)");

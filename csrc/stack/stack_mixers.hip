@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+
 #include "stack_device.h"
 #include "stack_ops.h"
 
@@ -922,6 +924,96 @@ __global__ __launch_bounds__(256) void moe_route_scores_kernel(MoeParams P) {
   }
   T* hm = (T*)P.hmid + (long long)b * P.ld_hmid + P.top * P.F;
   for (int f = threadIdx.x; f < P.Fs; f += 256) st(hm + f, silu(row[P.off_sgate + f]) * row[P.off_sup + f]);
+}
+// ---- a few rows (decode steps): routing and the routed and shared activations in one launch, as the top-k router's
+// moe_route_experts_kernel. Grid (ff units / 4, row x (top + 1)); every wave routes its row itself with one router
+// output per lane (X + identity <= 64): softmax across the lanes, one wave maximum per group, `keep` rounds of "best
+// group", `top` rounds of "best output" (ties: the lower lane). Block (0, row, 0) records ids, weights and idw.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_scores_experts_kernel(MoeParams P, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int b = blockIdx.y / (P.top + 1), jj = blockIdx.y % (P.top + 1);
+  const float* row = P.proj + (long long)b * P.ld;
+  T* hm = (T*)P.hmid + (long long)b * P.ld_hmid;
+  if (jj == P.top) {  // shared expert
+    if (f < P.Fs && lane == 0) st(hm + P.top * P.F + f, silu(row[P.off_sgate + f]) * row[P.off_sup + f]);
+    return;
+  }
+  const int NR = P.X + P.identity;
+  const bool has = lane < NR;
+  const float z = has ? row[P.off_router + lane] : -INFINITY;
+  const float zmax = wave_max(z);  // (every lane takes part in a wave reduction: never inside a lane condition)
+  const float ex = has ? expf(z - zmax) : 0.f;
+  const float sc = ex / wave_sum(ex);
+  float ch = has ? sc + P.router_b[lane] : -INFINITY;
+  if (P.group_count > 1) {
+    const int per = NR / P.group_count, mine = has ? lane / per : -1;
+    float gmax = -INFINITY;  // the largest choice score of this lane's group
+    for (int gi = 0; gi < P.group_count; ++gi) {
+      const float v = wave_max(mine == gi ? ch : -INFINITY);
+      if (mine == gi) gmax = v;
+    }
+    bool kept = false;
+    float gm = has ? gmax : -INFINITY;
+    for (int q = 0; q < P.group_keep; ++q) {
+      const float best = wave_max(gm);
+      const int who = max(0, __ffsll((unsigned long long)__ballot(gm == best)) - 1);  // lowest lane of the best group
+      const int gsel = who / per;
+      if (mine == gsel) {
+        kept = true;
+        gm = -INFINITY;
+      }
+    }
+    if (!kept) ch = -INFINITY;
+  }
+  int e = -1;
+  float idw = 0.f;
+  const bool rec = threadIdx.x < 64 && blockIdx.x == 0 && jj == 0;  // the wave that records the row's routing
+  for (int q = 0; q < P.top; ++q) {
+    const float mx = wave_max(ch);
+    const bool any = mx != -INFINITY;
+    const int who = max(0, __ffsll((unsigned long long)__ballot(ch == mx && has)) - 1);
+    const float w = __shfl(sc, who, 64);
+    const bool real = any && who < P.X;
+    if (q == jj) e = real ? who : -1;
+    if (any && !real) idw += w;
+    if (rec && lane == 0) {
+      P.eids[(long long)b * P.ld_top + q] = real ? who : 0;
+      P.ew[(long long)b * P.ld_top + q] = real ? w : 0.f;
+    }
+    if (lane == who) ch = -INFINITY;
+  }
+  if (rec && lane == 0) {
+    P.idw[b] = idw;
+    if (P.Fs > 0) P.sgate[b] = 1.f;
+  }
+  if (f >= P.F) return;
+  if (e < 0) {  // an identity output (or none): its place carries weight 0, and a finite activation
+    if (lane == 0) st(hm + jj * P.F + f, 0.f);
+    return;
+  }
+  const T* x = (const T*)P.h + (long long)b * P.E;
+  const T* wg = (const T*)P.w_gu + ((long long)e * 2 * P.F + f) * P.E;
+  const T* wu = wg + (long long)P.F * P.E;
+  const float gate = wave_dot<T>(wg, x, P.E, lane, vec != 0);
+  const float up = wave_dot<T>(wu, x, P.E, lane, vec != 0);
+  if (lane == 0) st(hm + jj * P.F + f, silu(gate) * up);
+}
+bool moe_route_scores_fused_supported(const MoeParams& P) { return P.X + P.identity <= 64 && P.group_count <= 64; }
+void moe_route_scores_experts(const MoeParams& P, hipStream_t s) {
+  check(P.B > 0 && P.proj && P.eids && P.ew && P.idw && P.router_b && P.h && P.w_gu && P.hmid && moe_route_scores_fused_supported(P) &&
+            P.top > 0 && P.top <= MOE_MAX_TOP && P.group_count >= 1 && (P.X + P.identity) % P.group_count == 0 &&
+            P.group_keep >= 1 && P.group_keep <= P.group_count && (P.Fs == 0 || P.sgate),
+        "fused score router: operands or sizes (up to 64 router outputs)");
+  const dim3 grid((std::max(P.F, P.Fs) + 3) / 4, P.B * (P.top + 1));
+  if (P.f32)
+    hipLaunchKernelGGL(moe_route_scores_experts_kernel<float>, grid, dim3(256), 0, s, P,
+                       (int)(vec_ok<float>(P.h, P.E, P.E) && vec_ok<float>(P.w_gu, P.E, P.E)));
+  else
+    hipLaunchKernelGGL(moe_route_scores_experts_kernel<bf16>, grid, dim3(256), 0, s, P,
+                       (int)(vec_ok<bf16>(P.h, P.E, P.E) && vec_ok<bf16>(P.w_gu, P.E, P.E)));
+  launched("moe_route_scores_experts");
 }
 void moe_route_scores(const MoeParams& P, hipStream_t s) {
   check(P.B > 0 && P.proj && P.eids && P.ew && P.idw && P.router_b && P.X + P.identity <= ROUTE_MAX && P.top > 0 &&

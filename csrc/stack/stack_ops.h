@@ -153,6 +153,9 @@ void moe_route(const MoeParams& P, hipStream_t s);   // top-k ids + softmax weig
 // chosen scores (not renormalised); leaves eids / ew / sgate (= 1) / the shared activation as moe_route does, so
 // moe_experts, moe_down and moe_grouped follow unchanged
 void moe_route_scores(const MoeParams& P, hipStream_t s);
+// a few rows (decode steps): the same routing and the routed and shared activations (moe_experts' work) in one launch
+void moe_route_scores_experts(const MoeParams& P, hipStream_t s);
+bool moe_route_scores_fused_supported(const MoeParams& P);
 void moe_experts(const MoeParams& P, hipStream_t s); // gate/up + activation of the routed experts -> hmid
 void moe_down(const MoeParams& P, hipStream_t s);    // y = sum_j w_j down_j(hmid_j) + sgate * shared_down(hmid_s)
 // a few rows (decode steps): routing + routed and shared activations in one launch, then the experts' down

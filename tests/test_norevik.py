@@ -69,6 +69,7 @@ MECHANISMS = {
     "moe_plain_top1": [(nc.mlstm(), nc.moe(experts=5, top=1, identity=0, groups=(1, 1), shared_ff=0))],
     "moe_all_groups_kept_identity_only_group": [(nc.mlstm(), nc.moe(experts=6, top=4, identity=3, groups=(3, 3), shared_ff=8))],
     "moe_one_group_kept": [(nc.mlstm(), nc.moe(experts=8, top=2, identity=0, groups=(4, 1)))],
+    "moe_more_choices_than_real_experts": [(nc.mlstm(), nc.moe(experts=2, top=4, identity=4, groups=(1, 1), shared_ff=16))],
 }
 
 
