@@ -59,9 +59,55 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(float* __restrict__ 
     if (hout) st(hout + r * E + i, v);
   }
 }
+// the same with the row held in registers (widths up to 256 * PN_REG): x and y are read once
+constexpr int PN_REG = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_add_reg_kernel(float* __restrict__ x, const float* __restrict__ y, int E,
+                                                                const float* __restrict__ w, const float* __restrict__ b,
+                                                                float eps, const float* __restrict__ idw, T* __restrict__ hout) {
+  __shared__ float red[4];
+  const long long r = blockIdx.x;
+  float* xr = x + r * E;
+  const float* yr = y + r * E;
+  const float iw = idw ? idw[r] : 0.f;
+  float xv[PN_REG], v[PN_REG];
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < PN_REG; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    xv[k] = i < E ? xr[i] : 0.f;
+    v[k] = i < E ? yr[i] + iw * xv[k] : 0.f;
+    sum += v[k];
+  }
+  const float mean = block_sum256(sum, red) / (float)E;
+  float sq = 0.f;
+#pragma unroll
+  for (int k = 0; k < PN_REG; ++k) {
+    const float d = threadIdx.x + 256 * k < E ? v[k] - mean : 0.f;
+    sq += d * d;
+  }
+  const float inv = 1.f / sqrtf(block_sum256(sq, red) / (float)E + eps);
+#pragma unroll
+  for (int k = 0; k < PN_REG; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    if (i < E) {
+      const float o = xv[k] + ((v[k] - mean) * inv * w[i] + b[i]);
+      xr[i] = o;
+      if (hout) st(hout + r * E + i, o);
+    }
+  }
+}
 void post_norm_add(float* x, const float* y, int rows, int E, const float* w, const float* b, float eps, const float* idw,
                    void* hout, int f32, hipStream_t s) {
   check(rows > 0 && E > 0 && x && y && w && b, "post_norm_add: bad operands");
+  if (E <= 256 * PN_REG) {
+    if (f32)
+      hipLaunchKernelGGL(post_norm_add_reg_kernel<float>, dim3(rows), dim3(256), 0, s, x, y, E, w, b, eps, idw, (float*)hout);
+    else
+      hipLaunchKernelGGL(post_norm_add_reg_kernel<bf16>, dim3(rows), dim3(256), 0, s, x, y, E, w, b, eps, idw, (bf16*)hout);
+    launched("post_norm_add");
+    return;
+  }
   if (f32)
     hipLaunchKernelGGL(post_norm_add_kernel<float>, dim3(rows), dim3(256), 0, s, x, y, E, w, b, eps, idw, (float*)hout);
   else
@@ -320,7 +366,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(ConvParams P, StepRows R
   // a sequence with ONE row in this step (a decode step): nobody else reads its window, so this block advances it
   const bool alone = nb == 0 && !(r + 1 < R.B && R.q_seq[r + 1] == seq);
   float* win = P.state + (long long)seq * P.state_stride;
-  for (int c = threadIdx.x; c < P.ch; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < P.ch; c += 256 * gridDim.y) {
     float acc = P.bias[c];
     const float cur = P.proj[(long long)r * P.ld + P.off_in + c];
     for (int j = 0; j < K; ++j) {
@@ -341,7 +387,7 @@ __global__ __launch_bounds__(256) void conv_window_kernel(ConvParams P, StepRows
   int n = 1;  // rows of the sequence in this step, up to taps - 1
   while (n < K - 1 && r - n >= 0 && R.q_seq[r - n] == seq) ++n;
   float* win = P.state + (long long)seq * P.state_stride;
-  for (int c = threadIdx.x; c < P.ch; c += 256)
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < P.ch; c += 256 * gridDim.y)
     for (int sidx = 0; sidx < K - 1; ++sidx) {
       const int back = K - 2 - sidx;
       win[(long long)sidx * P.ch + c] = back < n ? P.proj[(long long)(r - back) * P.ld + P.off_in + c]
@@ -351,10 +397,11 @@ __global__ __launch_bounds__(256) void conv_window_kernel(ConvParams P, StepRows
 void conv_silu(const ConvParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.proj && P.w && P.bias && P.out && P.ch > 0 && P.taps >= 1 && (P.taps == 1 || P.state),
         "conv_silu: bad operands");
-  hipLaunchKernelGGL(conv_silu_kernel, dim3(R.B), dim3(256), 0, s, P, R);
+  const dim3 grid(R.B, (P.ch + 255) / 256);  // a block per (row, 256 channels)
+  hipLaunchKernelGGL(conv_silu_kernel, grid, dim3(256), 0, s, P, R);
   launched("conv_silu");
   if (P.taps > 1 && R.B > 1) {  // a single row is alone in its sequence
-    hipLaunchKernelGGL(conv_window_kernel, dim3(R.B), dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL(conv_window_kernel, grid, dim3(256), 0, s, P, R);
     launched("conv_window");
   }
 }
