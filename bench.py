@@ -358,7 +358,8 @@ STACK_SIZES = {
 
 
 # the Norevik design at the same widths: latent attention x2, an mLSTM and a Mamba-2 layer, twice; the first layer's
-# feed-forward is dense, the others route 2 of 8 experts + 2 identity outputs in 2 groups, beside a shared expert
+# feed-forward is dense, the others route 2 of 8 experts + 4 identity outputs (4 groups, the best 2 kept), beside a
+# shared expert
 NOREVIK_SIZES = {
     "s": dict(E=1024, pattern="llxm" * 2, H=16, D=64, R=32, Dv=64, C=192, F=512, X=8, top=2, Fs=1024, dense=2048,
               mlstm=(8, 64, 128), mamba=(16, 64, 64, 1)),
@@ -384,7 +385,7 @@ def norevik_config(z: dict, vocab: int = 32000):
             m = MixerSpec(kind=MIX_MAMBA2, heads=h, kv_heads=g, dim=n, vdim=dv, state=n, groups=g, conv=4, norm_groups=g)
         f = (MoESpec(kind=FF_DENSE, ff=z["dense"]) if i == 0 else
              MoESpec(kind=FF_MOE, route=ROUTE_SCORE_GROUPS, experts=z["X"], top=z["top"], ff=z["F"], shared_ff=z["Fs"],
-                     identity=2, group_count=2, group_keep=1, shared_gate=False))
+                     identity=4, group_count=4, group_keep=2, shared_gate=False))
         layers.append(LayerSpec(mixer=m, mlp=f))
     return StackConfig(arch="norevik", n_vocab=vocab, n_embd=z["E"], layers=layers, norm_eps=1e-5, block=BLOCK_POSTNORM,
                        embed_scale=float(z["E"]) ** 0.5)
