@@ -70,6 +70,44 @@ def check(got, want, dtype, what=""):
             f"{what}: median row off by {np.median(e):.3g}, nine in ten within {np.quantile(e, 0.9):.3g}"
 
 
+def random_config(rng):
+    """A configuration drawn at the scale of a small real model: 4-7 layers of any mixer in any order, widths 128-320,
+    head counts, ranks, rotated parts, taps, groups and routers of many shapes (rng: random.Random)."""
+    width = rng.choice([128, 160, 224, 256, 320])
+
+    def lat():
+        R = rng.choice([0, 8, 16, 24, 32])
+        return latent(heads=rng.choice([2, 4, 5, 8]), dim=rng.choice([32, 48, 64, 96]), rot_dim=R, vdim=rng.choice([32, 48, 64, 80]),
+                      kv_rank=rng.choice([48, 64, 80, 128, 160]), scale=rng.choice([0.08, 0.15, 0.3]),
+                      rot_dims=(rng.choice([R, max(0, R - 8)]) if R else 0), base=rng.choice([1e4, 1e6]))
+
+    def ml():
+        return mlstm(heads=rng.choice([2, 3, 4, 8]), dim=rng.choice([16, 32, 48, 64]), vdim=rng.choice([24, 32, 64, 96]),
+                     cap=rng.choice([8.0, 12.0, 20.0]))
+
+    def mb():
+        G = rng.choice([1, 2, 4])
+        H = G * rng.choice([1, 2, 4])
+        return mamba(heads=H, vdim=rng.choice([16, 32, 64]), state=rng.choice([16, 32, 64, 128]), groups=G,
+                     conv=rng.choice([2, 3, 4]), norm_groups=rng.choice([1, G, H]))
+
+    def ff():
+        k = rng.random()
+        if k < 0.2:
+            return None
+        if k < 0.4:
+            return dense(rng.choice([256, 384, 512]))
+        gc, per = rng.choice([1, 2, 3, 4]), rng.choice([2, 3, 4])
+        nr = gc * per
+        ident = rng.choice([0, 1, 2]) if nr > 3 else 0
+        keep = rng.randint(1, gc)
+        return moe(experts=nr - ident, top=rng.randint(1, min(4, keep * per)), ff=rng.choice([64, 96, 128]),
+                   shared_ff=rng.choice([0, 128, 192]), identity=ident, groups=(gc, keep))
+
+    layers = [(rng.choice([lat, ml, mb])(), ff()) for _ in range(rng.randint(4, 7))]
+    return config(layers, width=width, vocab=rng.choice([500, 777, 1024]), eps=rng.choice([1e-5, 1e-6]), embed_scale=width ** 0.5)
+
+
 class Model(_Model):
     def oracle(self, toks):
         z, trail = oracle.forward(self.json, self.tensors, toks)

@@ -413,3 +413,29 @@ def test_matrix_core_attention_matches_twin(tmp_path, rank, rot):
     assert np.median(e) < 5e-3 and e.max() < 3e-2, f"HIP against twin: median {np.median(e):.3g}, worst {e.max():.3g}"
     e = nc.rel_err(b, want)
     assert np.median(e) < 2e-2 and e.max() < 0.1, f"HIP against the plain implementation: median {np.median(e):.3g}, worst {e.max():.3g}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at the scale of a small real model, a prompt of 700 tokens in portions of 64 and a tail of
+    single tokens against the whole prompt in one step and against the plain implementation, float32; bfloat16 against
+    the twin (the same rounding points: the two must be much closer to each other than either is to float64)."""
+    import random
+    cfg = nc.random_config(random.Random(100 + seed))
+    m = nc.Model(tmp_path, cfg, seed=seed)
+    n = 700
+    toks = nc.tokens(n, cfg.n_vocab, seed=seed)
+    want, _ = m.oracle(toks)
+    r = m.runner("cuda", "float32", max_batch=512, kv_tokens=1536)
+    cuts = list(range(64, n - 40, 64)) + [n - 37] + list(range(n - 36, n + 1))
+    for what, got in (("portions", nc.run_cuts(r, toks, cuts)), ("whole", nc.run_cuts(r, toks, [n]))):
+        e = nc.rel_err(got, want)  # stacks of up to seven layers: the odd ill-conditioned row may reach 1e-2
+        assert np.isfinite(got).all() and np.median(e) < 5e-5 and np.quantile(e, 0.99) < 1e-3 and e.max() < 2e-2, \
+            f"{what}: median {np.median(e):.3g}, 99 in 100 within {np.quantile(e, 0.99):.3g}, worst row {int(e.argmax())} by {e.max():.3g}"
+    short = toks[:300]
+    a = nc.run_cuts(m.runner("cpu", "bfloat16", max_batch=512, kv_tokens=512), short, [300])
+    b = nc.run_cuts(m.runner("cuda", "bfloat16", max_batch=512, kv_tokens=512), short, [64, 128, 192, 256, 298, 299, 300])
+    e = nc.rel_err(b, a)
+    assert np.isfinite(b).all() and np.median(e) < 0.04 and np.quantile(e, 0.9) < 0.2, \
+        f"bfloat16 HIP against twin: median {np.median(e):.3g}, nine in ten within {np.quantile(e, 0.9):.3g}"
